@@ -37,6 +37,10 @@ class PagedSlot:
     block_table: torch.Tensor      # int32 [max_rows, table_width], on the device
     block_size: int
     window: Optional[int]
+    # with pooled blocks (``PagedKV.pool``): the slot of the blocks' mean keys and values (its pages hold
+    # ``block_size`` entries, entry b of a row stands for positions b * pool .. b * pool + pool - 1)
+    pooled: Optional["PagedSlot"] = None
+    pool: int = 0
 
 
 @dataclass
@@ -48,8 +52,10 @@ class StateSlot:
 class PagedGroup:
     """Cache slots with the same need: one allocator, one table, a pool pair per slot."""
 
-    def __init__(self, need: PagedKV, max_rows, table_width, block_size, num_blocks, dtype, device):
-        self.need, self.block_size, self.table_width = need, block_size, table_width
+    def __init__(self, need: PagedKV, max_rows, table_width, block_size, num_blocks, dtype, device, per=1):
+        """``per``: positions that one entry of a page stands for (1: a token; P: the mean of a block of P
+        tokens, which exists once the block is complete and is never given back before the row closes)."""
+        self.need, self.block_size, self.table_width, self.per = need, block_size, table_width, per
         self.allocator = BlockAllocator(num_blocks)
         # one row more than can be opened: the null row, whose entries all point at the null
         # page, stands in for the padding rows of a fixed-width (captured) decode step
@@ -60,7 +66,7 @@ class PagedGroup:
         self.first_live = [0] * max_rows
         # with a window that keeps the first positions visible: the blocks that hold them stay with the
         # row whatever the window has passed (a row then holds blocks 0 .. kept and first_live .. covered)
-        keep_first = getattr(need, "keep_first", 0) if need.window is not None else 0
+        keep_first = getattr(need, "keep_first", 0) if need.window is not None and per == 1 else 0
         self.kept_blocks = blocks_for(keep_first, block_size) if keep_first > 0 else 0
         self.dirty = set()
         # a latent is kept as one "head" of ``width`` elements, in one pool per slot
@@ -79,9 +85,13 @@ class PagedGroup:
     # -- pages a row needs / can drop ---------------------------------------------------------
     def droppable(self, row: int, next_start: int) -> int:
         """Logical blocks of ``row`` that no token at position >= next_start can see."""
-        if self.need.window is None:
+        if self.need.window is None or self.per > 1:
             return self.first_live[row]
         first_visible = max(0, next_start - self.need.window + 1)
+        pool = getattr(self.need, "pool", 0)
+        if pool:
+            # the block that holds next_start is not complete: its tokens stay until its mean is taken
+            first_visible = min(first_visible, next_start // pool * pool)
         return max(self.first_live[row], min(first_visible // self.block_size, self.covered[row]))
 
     def _held(self, row: int):
@@ -98,7 +108,7 @@ class PagedGroup:
         return len(self._held(row))
 
     def missing(self, row: int, new_len: int) -> int:
-        return max(0, blocks_for(new_len, self.block_size) - self.covered[row])
+        return max(0, blocks_for(new_len // self.per, self.block_size) - self.covered[row])
 
     def drop_behind(self, row: int, next_start: int):
         upto = self.droppable(row, next_start)
@@ -115,7 +125,7 @@ class PagedGroup:
         if n:
             lo = self.covered[row]
             if lo + n > self.table_width:
-                raise ValueError(f"{new_len} tokens need {lo + n} blocks, the table holds {self.table_width}")
+                raise ValueError(f"{new_len} tokens need {lo + n} pages, the table holds {self.table_width}")
             self.host_table[row, lo:lo + n] = self.allocator.alloc(n)
             self.covered[row] = lo + n
             self.dirty.add(row)
@@ -179,32 +189,68 @@ class CacheManager:
         self.table_width = blocks_for(max_len, block_size)
         self.groups: List[PagedGroup] = []
         self._slots = []
-        by_need = {}
+        self._by_need = {}
+        self._num_blocks = num_blocks
         for slot_id, need in enumerate(needs):
-            if isinstance(need, (PagedKV, PagedLatent)):
-                if getattr(need, "keep_first", 0) < 0:
-                    raise ValueError(f"cache slot {slot_id}: keep_first is not negative")
-                group = by_need.get(need)
-                if group is None:
-                    group = PagedGroup(need, max_rows, self.table_width, block_size, num_blocks,
-                                       dtype, device)
-                    by_need[need] = group
-                    self.groups.append(group)
-                group.add_slot(slot_id)
-                k, v = group.pools[slot_id]
-                self._slots.append(PagedSlot(k, v, group.table, block_size, need.window))
-            elif isinstance(need, RowState):
-                kinds = {"float32": torch.float32, "int32": torch.int32, "compute": dtype}
-                if need.dtype not in kinds:
-                    raise ValueError(f"cache slot {slot_id}: a row's state is one of {sorted(kinds)}, not {need.dtype!r}")
-                state = torch.zeros((max_rows + 1,) + tuple(need.shape), dtype=kinds[need.dtype], device=device)
-                self._slots.append(StateSlot(state))
-            elif need is None:
-                self._slots.append(None)
-            else:
-                raise TypeError(f"cache slot {slot_id}: unknown kind of need {need!r}")
+            try:
+                self._slots.append(self._make_slot(need))
+            except (TypeError, ValueError) as e:
+                raise type(e)(f"cache slot {slot_id}: {e}") from None
         self.scalars = RowScalars(max_rows)
         self._open = [False] * max_rows
+
+    def _group(self, key, need, num_blocks, per=1):
+        group = self._by_need.get(key)
+        if group is None:
+            table_width = self.table_width if per == 1 else blocks_for(self.max_len // per, self.block_size)
+            group = PagedGroup(need, self.max_rows, max(table_width, 1), self.block_size, num_blocks, self.dtype,
+                               self.device, per=per)
+            self._by_need[key] = group
+            self.groups.append(group)
+        return group
+
+    def _make_slot(self, need):
+        if isinstance(need, tuple):
+            # a mixer made of several mixers: one slot for each, in order
+            return tuple(self._make_slot(n) for n in need)
+        if isinstance(need, (PagedKV, PagedLatent)):
+            if getattr(need, "keep_first", 0) < 0:
+                raise ValueError("keep_first is not negative")
+            pool = getattr(need, "pool", 0)
+            if pool < 0 or (pool and (need.window is None or need.keep_first)):
+                raise ValueError("pooled blocks need a window, and no kept first positions")
+            group = self._group(need, need, self._num_blocks)
+            serial = len(group.pools)
+            group.add_slot(serial)
+            k, v = group.pools[serial]
+            slot = PagedSlot(k, v, group.table, self.block_size, need.window)
+            if pool:
+                # the means of the blocks: as many entries as the tokens' pages hold blocks, and a page more per
+                # row for the rounding
+                entries = self._num_blocks * self.block_size // pool
+                means = self._group(("means", need), need, blocks_for(entries, self.block_size) + self.max_rows, per=pool)
+                means.add_slot(serial)
+                mk, mv = means.pools[serial]
+                slot.pooled, slot.pool = PagedSlot(mk, mv, means.table, self.block_size, None), pool
+            return slot
+        if isinstance(need, RowState):
+            kinds = {"float32": torch.float32, "int32": torch.int32, "compute": self.dtype}
+            if need.dtype not in kinds:
+                raise ValueError(f"a row's state is one of {sorted(kinds)}, not {need.dtype!r}")
+            state = torch.zeros((self.max_rows + 1,) + tuple(need.shape), dtype=kinds[need.dtype], device=self.device)
+            return StateSlot(state)
+        if need is None:
+            return None
+        raise TypeError(f"unknown kind of need {need!r}")
+
+    def _state_slots(self):
+        def walk(slots):
+            for s in slots:
+                if isinstance(s, tuple):
+                    yield from walk(s)
+                elif isinstance(s, StateSlot):
+                    yield s
+        return walk(self._slots)
 
     # -- rows ------------------------------------------------------------------------------
     @property
@@ -224,9 +270,8 @@ class CacheManager:
             raise RuntimeError(f"all {self.max_rows} rows are open")
         self._open[row] = True
         self.scalars.clear(row)
-        for s in self._slots:
-            if isinstance(s, StateSlot):
-                s.state[row].zero_()
+        for s in self._state_slots():
+            s.state[row].zero_()
         return row
 
     def close_row(self, row: int):
@@ -249,9 +294,8 @@ class CacheManager:
             g.covered[dst], g.covered[src] = g.covered[src], 0
             g.first_live[dst], g.first_live[src] = g.first_live[src], 0
             g.dirty.update((src, dst))
-        for s in self._slots:
-            if isinstance(s, StateSlot):
-                s.state[dst].copy_(s.state[src])
+        for s in self._state_slots():
+            s.state[dst].copy_(s.state[src])
         self.scalars.move(src, dst)
         self._open[dst], self._open[src] = True, False
 
@@ -293,7 +337,7 @@ class CacheManager:
         """Tokens one request can hold if it has the whole pool of every group."""
         if not self.groups:
             return self.max_len
-        return min(self.max_len, min(g.allocator.num_blocks for g in self.groups) * self.block_size)
+        return min(self.max_len, min(g.allocator.num_blocks * g.per for g in self.groups) * self.block_size)
 
     def reserve(self, row: int, new_len: int):
         """Make sure every group holds the pages for positions up to ``new_len`` of

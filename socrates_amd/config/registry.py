@@ -12,6 +12,7 @@ import json
 from pathlib import Path
 
 from .mitisun import MitisunConfig
+from .pozalorn import PozalornConfig
 from .qwen3 import ConfigError, Qwen3Config
 from .tedulorn import TedulornConfig
 
@@ -100,3 +101,4 @@ def load_preset(name: str):
 register_architecture("Qwen3ForCausalLM", Qwen3Config)
 register_architecture("Mitisun", MitisunConfig)
 register_architecture("Tedulorn", TedulornConfig)
+register_architecture("Pozalorn", PozalornConfig)

@@ -103,12 +103,38 @@ class PairRopeSpec:
     of a vector are one pair, turned by position * base ** (-2i / dims); the rest passes."""
     dims: int
     base: float
+    # (factor, low, high, original): a frequency whose wavelength is longer than original / low is divided
+    # by factor, one whose wavelength is shorter than original / high stays, and between the two, with
+    # s = (original / wavelength - low) / (high - low), it becomes (1 - s) f / factor + s f. None: no stretch.
+    stretch: Optional[Tuple[float, float, float, float]] = None
 
     def __post_init__(self):
         if self.dims < 2 or self.dims % 2:
             raise ValueError(f"a rotation over pairs needs an even number of dimensions, not {self.dims}")
         if not self.base > 0:
             raise ValueError("the rotation's base must be positive")
+        if self.stretch is not None:
+            factor, low, high, original = self.stretch
+            if not (factor > 0 and original > 0 and high > low > 0):
+                raise ValueError(f"stretch (factor, low, high, original) = {self.stretch}: factor and original are "
+                                 "positive and high lies above low")
+
+    def frequencies(self):
+        """The dims / 2 frequencies as Python floats (double precision)."""
+        import math
+        out = []
+        for i in range(self.dims // 2):
+            f = self.base ** (-2.0 * i / self.dims)
+            if self.stretch is not None:
+                factor, low, high, original = self.stretch
+                wave = 2.0 * math.pi / f
+                if wave > original / low:
+                    f = f / factor
+                elif wave >= original / high:
+                    t = (original / wave - low) / (high - low)
+                    f = (1.0 - t) * f / factor + t * f
+            out.append(f)
+        return out
 
 
 @dataclass(frozen=True)
@@ -346,6 +372,128 @@ class TokenSideSpec:
 
 
 @dataclass(frozen=True)
+class WindowAttentionSpec:
+    """Grouped-query softmax attention over a sliding window, with what designs put around it.
+
+    q, k [heads x ``head_dim``], v [kv heads x ``v_dim``], each with a bias if ``qkv_bias``. ``qk_norm``:
+    "head" (RMS norm over each head, one gain of head_dim for all heads), "whole" (RMS norm over the whole
+    projection of q, and of k, with a gain of that size) or None. ``position`` turns interleaved pairs of
+    q and k. ``value_base`` = B: the value of position j is turned by j over pairs (2m, 2m + 1) of all v_dim
+    elements with the frequencies B^(-2m / v_dim), and cached so; a head's result at position i is turned
+    back by i (None: values as they are). A query at position i sees key j with
+    0 <= i - j < ``window`` (None: all j <= i) and, with ``pool`` = P > 0, one mean key and mean value (of
+    what the cache holds) for every block bP .. bP + P - 1 with bP + P - 1 <= i - window, in the same
+    softmax. ``sinks``: a stored number per head whose exponential joins the softmax's denominator."""
+    hidden: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    v_dim: int
+    scale: float
+    eps: float
+    qk_norm: Optional[str] = None
+    position: Optional[PairRopeSpec] = None
+    window: Optional[int] = None
+    pool: int = 0
+    sinks: bool = False
+    qkv_bias: bool = False
+    o_bias: bool = False
+    value_base: Optional[float] = None
+
+    def __post_init__(self):
+        if self.n_heads < 1 or self.n_kv_heads < 1 or self.n_heads % self.n_kv_heads:
+            raise ValueError(f"n_heads {self.n_heads} is not a multiple of n_kv_heads {self.n_kv_heads}")
+        if not 1 <= self.head_dim <= 256 or not 1 <= self.v_dim <= 256:
+            raise ValueError(f"head sizes {self.head_dim} and {self.v_dim}: the attention kernels take up to 256")
+        if self.qk_norm not in (None, "head", "whole"):
+            raise ValueError(f"qk_norm {self.qk_norm!r}: head, whole or None")
+        if self.window is not None and self.window < 1:
+            raise ValueError("window must be at least 1")
+        if self.pool < 0 or (self.pool and self.window is None):
+            raise ValueError("pooled blocks lie before a window: pool needs a window and is not negative")
+        if self.position is not None and self.position.dims > self.head_dim:
+            raise ValueError(f"the rotation covers {self.position.dims} dimensions, a head has {self.head_dim}")
+        if self.value_base is not None and (not self.value_base > 0 or self.v_dim % 2):
+            raise ValueError("turned values need a positive base and an even v_dim")
+        if not self.scale > 0:
+            raise ValueError("scale must be positive")
+
+    @property
+    def cache_width(self) -> int:
+        """Elements per cached key and per cached value: the larger of the two sizes, padded to the
+        kernels' step."""
+        return (max(self.head_dim, self.v_dim) + 15) // 16 * 16
+
+
+@dataclass(frozen=True)
+class GatedLinearAttentionSpec:
+    """Linear attention with a decay per key channel that depends on the token: q = Wq h * head_dim^-1/2,
+    k = Wk h, v = Wv h; alpha = sigmoid(Wa2 (Wa1 h) + b)^(1 / tau) [heads x head_dim];
+    S <- diag(alpha) S + k v^T, o = S^T q per head; each head's o RMS-normed with one gain of v_dim for
+    all heads, times silu(Wg h), then the output projection. The state is float32 and starts at zero.
+    ``decay_rank`` 0: whatever Wa1 holds on disk."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    v_dim: int
+    tau: float
+    eps: float
+    decay_rank: int = 0
+
+    def __post_init__(self):
+        if self.n_heads < 1 or not 1 <= self.head_dim <= 256 or self.v_dim < 1:
+            raise ValueError(f"gated linear attention: {self.n_heads} heads of {self.head_dim} (1 to 256) and {self.v_dim}")
+        if not self.tau > 0:
+            raise ValueError("tau must be positive")
+
+
+@dataclass(frozen=True)
+class LightningAttentionSpec:
+    """Linear attention with a fixed decay per head over activated projections: q = silu(Wq h),
+    k = silu(Wk h), v = silu(Wv h); S <- decay_h S + k v^T, o = S^T q; the heads together RMS-normed with
+    a gain, times sigmoid(Wg h), then the output projection. The state is float32 and starts at zero."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    v_dim: int
+    decays: Tuple[float, ...]
+    eps: float
+
+    def __post_init__(self):
+        if self.n_heads < 1 or len(self.decays) != self.n_heads:
+            raise ValueError(f"lightning attention: {len(self.decays)} decays for {self.n_heads} heads")
+        if not 1 <= self.head_dim <= 256 or self.v_dim < 1:
+            raise ValueError(f"lightning attention: heads of {self.head_dim} (1 to 256) and {self.v_dim}")
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Two mixers side by side on the same input: ``left_scale`` * left(h) + ``right_scale`` * right(h);
+    their tensors lie under ``left.`` and ``right.``, and each keeps its own cache or state."""
+    left: object
+    right: object
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+
+
+@dataclass(frozen=True)
+class GeluGLUSpec:
+    """y = Wd(gelu_tanh(Wg x) * (Wu x)), no bias;
+    gelu_tanh(z) = 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))."""
+    hidden: int
+    intermediate: int
+
+
+@dataclass(frozen=True)
+class DepthAverageSpec:
+    """What goes on from layer ``index``: sum over j = 0 .. index + 1 of w[j] X_j, with X_0 the embedding
+    output, X_(j+1) layer j's own result (before this sum) and w a stored vector of index + 2 numbers.
+    ``n_layers``: how many layers the model has (a step keeps that many results and one)."""
+    index: int
+    n_layers: int
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One layer: which mixer, feed-forward and norms, how they are arranged,
     and the prefix its tensors carry on disk.
@@ -374,8 +522,12 @@ class BlockSpec:
     # For the arrangement "prenorm_side": prenorm, then x <- x + side(x) on the stream itself (``side``
     # None: none); ``ffn`` None: the layer has no feed-forward and no norm2.
     side: object = None
+    # For the arrangement "postnorm_depth": x <- x + norm1(mixer(x)); x <- x + norm2(ffn(x)) (the parts read
+    # the stream itself, the norms act on their results; ``ffn`` None: no feed-forward and no norm2); then
+    # what goes on is ``depth``'s weighted sum of the embedding output and all layers' results so far.
+    depth: object = None
 
-    ROLES = ("norm1", "mixer", "norm2", "ffn", "post_norm1", "post_norm2", "gate1", "gate2", "side")
+    ROLES = ("norm1", "mixer", "norm2", "ffn", "post_norm1", "post_norm2", "gate1", "gate2", "side", "depth")
 
     def name_of(self, role: str) -> str:
         return self.prefix + dict(self.names)[role]

@@ -8,8 +8,8 @@ branch output un-added ("pending") and the next norm adds it.
 
 from __future__ import annotations
 
-from ..config.specs import BlockSpec
-from .registry import build_part, tensors_of
+from ..config.specs import BlockSpec, DepthAverageSpec
+from .registry import TensorDecl, build_part, register_part, tensors_of
 
 _ARRANGEMENTS = {}
 
@@ -215,6 +215,72 @@ class SideInputBlock:
         return None if rows is None else Normed(rows)
 
 
+class DepthAverage:
+    """Holds the weights w [index + 2] of what goes on from a layer: sum_j w[j] X_j over the embedding output
+    X_0 and the results X_1 .. X_(index+1) of the layers so far."""
+
+    @staticmethod
+    def tensors(spec):
+        return {"": TensorDecl((spec.index + 2,), "vector")}
+
+    def __init__(self, spec, tensors, ops):
+        self.spec, self.weights = spec, tensors[""]
+
+
+class DepthAverageBlock:
+    """Norms on the results only, and a weighted sum over depth at the end: x <- x + norm1(mixer(x));
+    x <- x + norm2(ffn(x)) (a layer may have no feed-forward), mixer and feed-forward reading the stream
+    itself; that x is the layer's result X_(i+1), and what goes on is sum_j w[j] X_j over the embedding
+    output and all layers' results so far. The results are kept in float32 for the length of the step
+    (``ctx.carry``: one tensor [layers + 1, N, d] that the first block of a step makes). One kernel norms
+    a branch's result, adds it to the stream and casts the sum for the part that reads it next; one more
+    files the layer's result, takes the weighted sum and casts it for the next layer's mixer."""
+    chains = True
+    _CARRY = "results by depth"
+
+    def __init__(self, spec: BlockSpec, weights, ops):
+        self.spec, self.ops = spec, ops
+        built = {}
+        for role in ("norm1", "mixer", "norm2", "ffn", "depth"):
+            sub = getattr(spec, role)
+            built[role] = None if sub is None else build_part(sub, _sub_tensors(spec, role, weights), ops)
+        # (the norms are not called norm1 / norm2 here: a block of another arrangement in front of this one
+        # would take a ``norm1`` for a norm on this block's input)
+        self.post1, self.mixer, self.post2, self.ffn, self.depth = (built[r] for r in ("norm1", "mixer", "norm2", "ffn", "depth"))
+        if self.ffn is not None and self.post2 is None:
+            raise ValueError("a feed-forward needs the norm behind it")
+        if self.depth is None:
+            raise ValueError("this arrangement ends with a weighted sum over depth")
+        parts = (self.post1, self.mixer, self.post2, self.ffn)
+        self.capturable = all(getattr(p, "capturable", True) for p in parts if p is not None)
+
+    def reserve(self, n_positions):
+        for part in (self.mixer, self.ffn):
+            if hasattr(part, "reserve"):
+                part.reserve(n_positions)
+
+    def forward(self, residual, pending, ctx, slot, write=True, nxt=None):
+        ops = self.ops
+        depth = self.depth.spec
+        # the stream in the compute dtype, for the mixer: the block before has left it, or it is cast here
+        # (with whatever that block left un-added)
+        x = pending.rows if isinstance(pending, Normed) else ops.add_cast(residual, pending)
+        if depth.index == 0:
+            # the first layer of a step files the embedding output as X_0
+            ctx.carry[self._CARRY] = ops.depth_begin(residual, depth.n_layers + 1)
+        kept = ctx.carry[self._CARRY]
+        gain, eps = self.post1.fusable()
+        x = ops.norm_add_cast(residual, self.mixer.forward(x, ctx, slot, write), gain, eps, cast=self.ffn is not None)
+        if self.ffn is not None:
+            gain, eps = self.post2.fusable()
+            ops.norm_add_cast(residual, self.ffn.forward(x, ctx), gain, eps, cast=False)
+        rows = ops.depth_average(residual, kept, depth.index + 1, self.depth.weights, cast=isinstance(nxt, DepthAverageBlock))
+        return None if rows is None else Normed(rows)
+
+
+register_arrangement("postnorm_depth", DepthAverageBlock)
 register_arrangement("prenorm", PreNormBlock)
 register_arrangement("prenorm_side", SideInputBlock)
 register_arrangement("sandwich", SandwichBlock)
+
+register_part(DepthAverageSpec, DepthAverage)

@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import torch
 
-from ..config.specs import ClampedGLUSpec, ReluSquaredSpec, SigmoidGateSpec, SwiGLUSpec
+from ..config.specs import ClampedGLUSpec, GeluGLUSpec, ReluSquaredSpec, SigmoidGateSpec, SwiGLUSpec
 from .registry import TensorDecl, register_part
 
 
@@ -90,6 +90,24 @@ class ReluSquared:
         return self.ops.linear(self.ops.relu_squared(self.ops.linear(x, self.w_up)), self.w_down)
 
 
+class GeluGLU:
+    """y = Wd(gelu_tanh(Wg x) * (Wu x))."""
+
+    @staticmethod
+    def tensors(spec: GeluGLUSpec):
+        return {"gate": TensorDecl((spec.intermediate, spec.hidden)), "up": TensorDecl((spec.intermediate, spec.hidden)),
+                "down": TensorDecl((spec.hidden, spec.intermediate))}
+
+    def __init__(self, spec: GeluGLUSpec, tensors, ops):
+        self.spec, self.ops = spec, ops
+        self.w_gate_up = torch.cat([tensors["gate"], tensors["up"]], dim=0).contiguous()      # rows [gate | up]
+        self.w_down = tensors["down"]
+
+    def forward(self, x, ctx=None):
+        act = self.ops.glu_gelu(self.ops.linear(x, self.w_gate_up), self.spec.intermediate)
+        return self.ops.linear(act, self.w_down)
+
+
 class SigmoidGate:
     """Holds W [dim, dim] and b [dim] of sigmoid(W h + b); the block computes it where it closes
     a branch."""
@@ -106,3 +124,4 @@ register_part(SwiGLUSpec, SwiGLU)
 register_part(ClampedGLUSpec, ClampedGLU)
 register_part(SigmoidGateSpec, SigmoidGate)
 register_part(ReluSquaredSpec, ReluSquared)
+register_part(GeluGLUSpec, GeluGLU)

@@ -63,11 +63,17 @@ class TensorDecl:
 class PagedKV:
     """A mixer that keeps keys and values of every position (or a window of them) in pages.
     ``keep_first``: with a window, the positions below it stay visible to every later token, so
-    the pages that hold them are never given back before the row closes."""
+    the pages that hold them are never given back before the row closes. ``pool`` = P > 0, with a window:
+    beside the tokens' pages the slot keeps one mean key and value per block of P positions, in pages of
+    their own (entry b of a row stands for positions bP .. bP + P - 1), and a token's page is held until the
+    block of its last position is complete, so that the means can be taken from the pages.
+
+    A mixer made of several mixers names a tuple of needs; its slot is then the tuple of their slots."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     keep_first: int = 0
+    pool: int = 0
 
 
 @dataclass(frozen=True)

@@ -148,6 +148,16 @@ class TorchKernels:
             offs = torch.as_tensor(idx % bs, device=q.device)
             k = slot.k[pages, :, offs].to(self.acc)          # [n, Hkv, D]
             v = slot.v[pages, :, offs].to(self.acc)
+            if terms.get("pooled") is not None and window is not None:
+                # the means of the blocks that lie wholly before the window, in front of the window's keys
+                means, per = terms["pooled"].pooled, terms["pooled"].pool
+                blocks = np.arange(max(0, (p - window + 1) // per))
+                mtable = means.block_table.cpu().numpy()
+                mp = torch.as_tensor(mtable[row, blocks // bs].astype(np.int64), device=q.device)
+                mo = torch.as_tensor(blocks % bs, device=q.device)
+                k = torch.cat([means.k[mp, :, mo].to(self.acc), k], dim=0)
+                v = torch.cat([means.v[mp, :, mo].to(self.acc), v], dim=0)
+                idx = np.concatenate([blocks, idx])
             qt = q[t].to(self.acc).view(Hkv, G, D)
             s = torch.einsum("hgd,nhd->hgn", qt, k) * scale
             if terms.get("slopes") is not None:
@@ -252,11 +262,11 @@ class TorchKernels:
             state[row, offset:offset + H * Ns * P] = S.reshape(-1).to(state.dtype)
         return out.reshape(N, inner).to(torch.float32 if A == torch.float32 else A)
 
-    def gated_group_norm(self, y, z, gain, groups, eps, gate_first=True):
+    def gated_group_norm(self, y, z, gain, groups, eps, gate_first=True, sigmoid=False):
         A = self.acc
         N, inner = y.shape
         zz = z[:, :inner].to(A)
-        gate = zz * torch.sigmoid(zz)
+        gate = torch.sigmoid(zz) if sigmoid else zz * torch.sigmoid(zz)
         y = y.to(A) * gate if gate_first else y.to(A)
         y = y.view(N, groups, inner // groups)
         y = y / torch.sqrt(y.pow(2).mean(-1, keepdim=True) + eps)
@@ -414,6 +424,109 @@ class TorchKernels:
         if delta is not None:
             residual += (delta.sum(0) if delta.dim() == 3 else delta).to(residual.dtype)
         return residual.to(self.dtype)
+
+    # -- norms on results with a weighted sum over depth; window attention with pooled blocks; linear attention ----
+    def depth_begin(self, residual, total):
+        kept = torch.zeros((total,) + tuple(residual.shape), dtype=residual.dtype, device=residual.device)
+        kept[0] = residual
+        return kept
+
+    def norm_add_cast(self, residual, y, gain, eps, cast=True):
+        residual += self._norm(y, gain, eps).to(residual.dtype)
+        return residual.to(self.dtype) if cast else None
+
+    def depth_average(self, residual, kept, count, weights, cast=True):
+        kept[count] = residual
+        w = weights.to(self.acc).view(-1, 1, 1)
+        residual.copy_((w[:count + 1] * kept[:count + 1].to(self.acc)).sum(0).to(residual.dtype))
+        return residual.to(self.dtype) if cast else None
+
+    def window_prepare(self, x, cols, Hq, Hkv, D, Dv, P, bias, q_gain, k_gain, norm, eps, inv_freq, rotary_dim, value_freq,
+                       positions, token_rows, slot):
+        A = self.acc
+        N = x.shape[0]
+        cq, ck, cv = cols
+        q, k, v = x[:, cq:cq + Hq * D].to(A), x[:, ck:ck + Hkv * D].to(A), x[:, cv:cv + Hkv * Dv].to(A)
+        if bias is not None:
+            b = bias.to(A)
+            q, k, v = q + b[cq:cq + Hq * D], k + b[ck:ck + Hkv * D], v + b[cv:cv + Hkv * Dv]
+        if norm == "whole":
+            q, k = self._norm(q, q_gain, eps), self._norm(k, k_gain, eps)
+        q, k, v = q.reshape(N, Hq, D), k.reshape(N, Hkv, D), v.reshape(N, Hkv, Dv)
+        if norm == "head":
+            q, k = self._norm(q, q_gain, eps), self._norm(k, k_gain, eps)
+        if rotary_dim:
+            q = self._turn_pairs(q, positions, inv_freq)
+            k = self._turn_pairs(k, positions, inv_freq)
+        if value_freq is not None:
+            v = self._turn_pairs(v, positions, value_freq)
+        out = torch.zeros((N, Hq, P), dtype=self.dtype, device=x.device)
+        out[..., :D] = q.to(self.dtype)
+        kp = torch.zeros((N, Hkv, P), dtype=slot.k.dtype, device=x.device)
+        vp = torch.zeros((N, Hkv, P), dtype=slot.v.dtype, device=x.device)
+        kp[..., :D] = k.to(slot.k.dtype)
+        vp[..., :Dv] = v.to(slot.v.dtype)
+        self.kv_write(kp, vp, positions, token_rows, slot)
+        return out
+
+    def pool_blocks(self, slot, ctx):
+        """The means of the blocks whose last position is one of the step's, from the pages."""
+        per, bs, means = slot.pool, slot.block_size, slot.pooled
+        table, mtable = slot.block_table.cpu().numpy(), means.block_table.cpu().numpy()
+        ends = ctx.seq_ctx.cpu().tolist()
+        for i, (row, lo, hi) in enumerate(self._sequences(ctx)):
+            start = ends[i] - (hi - lo)
+            for b in range(start // per, ends[i] // per):
+                idx = np.arange(b * per, b * per + per)
+                pages = torch.as_tensor(table[row, idx // bs].astype(np.int64))
+                offs = torch.as_tensor(idx % bs)
+                page = int(mtable[row, b // bs])
+                means.k[page, :, b % bs] = slot.k[pages, :, offs].to(self.acc).mean(0).to(means.k.dtype)
+                means.v[page, :, b % bs] = slot.v[pages, :, offs].to(self.acc).mean(0).to(means.v.dtype)
+
+    def turn_back(self, o, H, P, Dv, value_freq, positions):
+        N = o.shape[0]
+        y = o.view(N, H, P)[..., :Dv].to(self.acc)
+        if value_freq is not None:
+            y = self._turn_pairs(y, -positions, value_freq)
+        return y.reshape(N, H * Dv).to(self.dtype)
+
+    def linear_attention(self, x, cols, H, D, Dv, q_scale, activate, decays, z, z_bias, tau, state, offset, ctx):
+        A = self.acc
+        N = x.shape[0]
+        cq, ck, cv = cols
+        q = x[:, cq:cq + H * D].reshape(N, H, D).to(A)
+        k = x[:, ck:ck + H * D].reshape(N, H, D).to(A)
+        v = x[:, cv:cv + H * Dv].reshape(N, H, Dv).to(A)
+        if activate:
+            q, k, v = q * torch.sigmoid(q), k * torch.sigmoid(k), v * torch.sigmoid(v)
+        q = q * q_scale
+        if z is not None:
+            decay = torch.exp(torch.nn.functional.logsigmoid(z.to(A) + z_bias.to(A)) / tau).view(N, H, D)
+        else:
+            decay = decays.to(A).view(1, H, 1).expand(N, H, D)
+        out = torch.empty((N, H, Dv), dtype=A, device=x.device)
+        for row, lo, hi in self._sequences(ctx):
+            S = state[row, offset:offset + H * D * Dv].to(A).view(H, D, Dv).clone()
+            for t in range(lo, hi):
+                S = decay[t].unsqueeze(-1) * S + k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
+                out[t] = torch.einsum("hk,hkv->hv", q[t], S)
+            state[row, offset:offset + H * D * Dv] = S.reshape(-1).to(state.dtype)
+        return out.reshape(N, H * Dv).to(torch.float32 if A == torch.float32 else A)
+
+    def scaled_sum(self, a, a_scale, b, b_scale, bias=None):
+        y = a.to(self.acc)
+        if bias is not None:
+            y = y + bias.to(self.acc)
+        y = a_scale * y
+        if b is not None:
+            y = y + b_scale * b.to(self.acc)
+        return y.to(torch.float32 if self.acc == torch.float32 else self.acc)
+
+    def glu_gelu(self, gate_up, ff):
+        z = gate_up[..., :ff].to(self.acc)
+        g = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        return (g * gate_up[..., ff:2 * ff].to(self.acc)).to(self.dtype)
 
     # -- sampling ----------------------------------------------------------------------------
     def argmax(self, logits):
