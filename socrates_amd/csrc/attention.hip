@@ -63,12 +63,28 @@ __device__ __forceinline__ void merge_partial(float& m, float& l, float (&a)[EPL
 //            contributes no value: the sum of weights gains exp(sinks[h] - max)
 //   keep_first  with a window: the keys at positions below keep_first stay visible to every later token,
 //            at their true positions (a token then walks those keys, then its window)
+//   pool     > 0, with a window: before its window a token sees one mean key and value for every block of
+//            pool positions that lies wholly before the window (block b if b * pool + pool - 1 <= p - window);
+//            entry b of the row's pages of means (mean_k, mean_v: pools of the cache's shape, with a table of
+//            their own) holds them. A token then walks those entries, then its window. Not with keep_first.
 struct ScoreTerms {
     float softcap;
     const float* sinks;
     const float* slopes;
     int keep_first;
+    const void* mean_k;
+    const void* mean_v;
+    const int* mean_table;
+    int mean_table_width;
+    int pool;
 };
+
+// How many entries a token at position p walks before its window (which starts at lo): kept first keys, or the
+// means of the blocks that lie wholly before the window.
+__device__ __forceinline__ int walk_prefix(const ScoreTerms& st, int p, int window, int lo) {
+    if (st.pool > 0) return window > 0 ? max(0, (p - window + 1) / st.pool) : 0;
+    return min(st.keep_first, lo);
+}
 
 template <typename T, int GC>
 __global__ void __launch_bounds__(256)
@@ -84,7 +100,7 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
     const int n = blockIdx.y, split = blockIdx.z;
     const int p = positions[n];
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
-    const int kf = min(st.keep_first, lo);             // kept first keys that lie before the window
+    const int kf = walk_prefix(st, p, window, lo);     // kept first keys (or means of blocks) that lie before the window
     // the token's keys in the order they are walked: the kept first ones, then lo .. p
     const int start = split * split_len;
     const int end = min(kf + p + 1 - lo, start + split_len);
@@ -93,6 +109,7 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
     const int tid = threadIdx.x;
     const int kg = tid / 16, l16 = tid % 16;           // key group 0..15, lane in the group
     const int* table = block_table + (size_t)token_rows[n] * table_width;
+    const int* mean_table = st.pool > 0 ? st.mean_table + (size_t)token_rows[n] * st.mean_table_width : table;
 
     // The group's queries, scaled, in registers: GC heads x EPL elements.
     float qr[GC][EPL];
@@ -123,11 +140,13 @@ paged_attn_token_kernel(const T* __restrict__ q, const T* __restrict__ k_pool,
 #pragma unroll
         for (int u = 0; u < KEYS_IN_FLIGHT; ++u) {
             if (base + 16 * u < end) {
-                const int key = base + 16 * u < kf ? base + 16 * u : base + 16 * u - kf + lo;
-                const int page = table[key / BS];
+                const bool before = base + 16 * u < kf;
+                const int key = before ? base + 16 * u : base + 16 * u - kf + lo;
+                const bool mean = before && st.pool > 0;           // entry `key` of the row's means
+                const int page = (mean ? mean_table : table)[key / BS];
                 const size_t off = ((size_t)page * Hkv * BS + (size_t)(key % BS)) * D + head_off;
-                VecLoad<T, EPL>::load(k_pool + off, kx[u]);
-                VecLoad<T, EPL>::load(v_pool + off, vx[u]);
+                VecLoad<T, EPL>::load((mean ? (const T*)st.mean_k : k_pool) + off, kx[u]);
+                VecLoad<T, EPL>::load((mean ? (const T*)st.mean_v : v_pool) + off, vx[u]);
             }
         }
 #pragma unroll
@@ -216,7 +235,7 @@ __global__ void paged_attn_reduce_kernel(const float* __restrict__ part_o,
     const int h = blockIdx.x, n = blockIdx.y;
     const int p = positions[n];
     const int lo = window > 0 ? max(0, p - window + 1) : 0;
-    const int np = min(n_splits, (min(st.keep_first, lo) + p + 1 - lo + split_len - 1) / split_len);
+    const int np = min(n_splits, (walk_prefix(st, p, window, lo) + p + 1 - lo + split_len - 1) / split_len);
     const size_t base = ((size_t)n * Hq + h) * n_splits;
     float M = st.sinks ? st.sinks[h] : -INFINITY;
     for (int s = 0; s < np; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
@@ -267,17 +286,22 @@ static int dispatch_token(int G, const void* q, const void* k_pool, const void* 
 // n_splits > 1 needs part_o [N, Hq, n_splits, D] and part_ml [N, Hq, n_splits, 2] (float32);
 // split s covers the keys s * split_len .. of each token's walk (the kept first keys, then its window).
 // softcap (0: none), sinks and slopes ([Hq] float32 each, or null) and keep_first (0: none): see
-// ScoreTerms. Any scale, also none or a negative one.
+// ScoreTerms; pool (0: none) with mean_k, mean_v [pages, Hkv, BS, D] and mean_table [rows, mean_table_width]: the
+// means of blocks before the window. Any scale, also none or a negative one.
 SOC_EXPORT int soc_paged_attention_tokens(const void* q, const void* k_pool, const void* v_pool,
                                           const int* block_table, int table_width,
                                           const int* token_rows, const int* positions, void* out,
                                           float* part_o, float* part_ml, int N, int Hq, int Hkv,
                                           int BS, float scale, int window, int split_len,
                                           int n_splits, int dtype, float softcap, const float* sinks,
-                                          const float* slopes, int keep_first, hipStream_t stream) {
+                                          const float* slopes, int keep_first, const void* mean_k,
+                                          const void* mean_v, const int* mean_table, int mean_table_width,
+                                          int pool, hipStream_t stream) {
     if (N <= 0) return 0;
     if (Hkv < 1 || Hq % Hkv || BS < 1 || n_splits < 1 || split_len < 1 || softcap < 0.f || keep_first < 0) return (int)hipErrorInvalidValue;
-    const ScoreTerms st{softcap, sinks, slopes, window > 0 ? keep_first : 0};
+    if (pool < 0 || (pool > 0 && (window <= 0 || keep_first > 0 || slopes || !mean_k || !mean_v || !mean_table)))
+        return (int)hipErrorInvalidValue;
+    const ScoreTerms st{softcap, sinks, slopes, window > 0 ? keep_first : 0, mean_k, mean_v, mean_table, mean_table_width, pool};
     if (n_splits > 1 && (!part_o || !part_ml)) return (int)hipErrorInvalidValue;
     if (N > 65535 || n_splits > 65535) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;

@@ -645,12 +645,12 @@ SOC_EXPORT int soc_causal_conv_silu(const void* x, int ldx, int col, int C, cons
 
 // ---- RMS norm in equal parts with a gate silu(z), in front of the norm or behind it ------------------------
 // y float32 [N, inner]; z the first `inner` columns of rows of ldz elements. Gate first: norm(y silu(z)) gain;
-// gate last: norm(y) gain silu(z). An item (part, token) is one wave's (four items to a workgroup), or, for
+// gate last: norm(y) gain silu(z). sigmoid_gate: the gate is sigmoid(z) in place of silu(z). An item (part, token) is one wave's (four items to a workgroup), or, for
 // parts of 512 elements and more, a whole workgroup's.
 template <typename T, bool GATE_FIRST, int WAVES>
 __global__ void __launch_bounds__(256)
 gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int ldz, const float* __restrict__ gain,
-                        int inner, int part, int n_items, float eps, T* __restrict__ out) {
+                        int inner, int part, int n_items, float eps, int sigmoid_gate, T* __restrict__ out) {
     __shared__ float scratch[16];
     constexpr int THREADS = WAVES * SOC_WAVE;
     const int item = WAVES == 1 ? blockIdx.x * (256 / SOC_WAVE) + threadIdx.x / SOC_WAVE : blockIdx.x;
@@ -661,20 +661,20 @@ gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, in
     float ss = 0.f;
     for (int c = c0 + lane; c < c0 + part; c += THREADS) {
         float v = y[(size_t)n * inner + c];
-        if (GATE_FIRST) { const float zz = to_float(z[(size_t)n * ldz + c]); v *= zz * soc_sigmoid(zz); }
+        if (GATE_FIRST) { const float zz = to_float(z[(size_t)n * ldz + c]); v *= sigmoid_gate ? soc_sigmoid(zz) : zz * soc_sigmoid(zz); }
         ss += v * v;
     }
     ss = WAVES == 1 ? wave_sum(ss) : block_sum(ss, scratch);
     const float inv = 1.f / sqrtf(ss / (float)part + eps);
     for (int c = c0 + lane; c < c0 + part; c += THREADS) {
         const float zz = to_float(z[(size_t)n * ldz + c]);
-        const float v = y[(size_t)n * inner + c] * zz * soc_sigmoid(zz);
+        const float v = y[(size_t)n * inner + c] * (sigmoid_gate ? soc_sigmoid(zz) : zz * soc_sigmoid(zz));
         out[(size_t)n * inner + c] = from_float<T>(v * inv * gain[c]);
     }
 }
 
 SOC_EXPORT int soc_gated_group_norm(const float* y, const void* z, int ldz, const float* gain, int N, int inner, int parts,
-                                    float eps, int gate_first, void* out, int dtype, hipStream_t stream) {
+                                    float eps, int gate_first, int sigmoid_gate, void* out, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
     if (parts < 1 || inner % parts || (long long)N * parts > 0x7fffffffLL) return (int)hipErrorInvalidValue;
     const int items = N * parts;
@@ -682,7 +682,7 @@ SOC_EXPORT int soc_gated_group_norm(const float* y, const void* z, int ldz, cons
     const dim3 grid(wide ? items : (items + 3) / 4);
 #define SOC_GGN(T, FIRST, WAVES)                                                                                              \
     hipLaunchKernelGGL((gated_group_norm_kernel<T, FIRST, WAVES>), grid, dim3(256), 0, stream, y, (const T*)z, ldz, gain, inner, \
-                       inner / parts, items, eps, (T*)out)
+                       inner / parts, items, eps, sigmoid_gate, (T*)out)
 #define SOC_GGN_T(T)                                                                                   \
     if (gate_first) { if (wide) SOC_GGN(T, true, 4); else SOC_GGN(T, true, 1); }                       \
     else { if (wide) SOC_GGN(T, false, 4); else SOC_GGN(T, false, 1); }

@@ -23,6 +23,7 @@ from ctypes import c_float, c_int, c_longlong, c_void_p
 import torch
 
 from .attention import Attention
+from .composite import Composite
 from .hybrid import Hybrid
 from .mixers import Mixers
 from .build import KernelBuildError, build_all, compile_library, load_library
@@ -35,7 +36,7 @@ __all__ = ["HipKernels", "KernelBuildError", "KernelError", "MAX_KEY_SPLITS", "N
            "compile_library", "load_library", "plan_key_splits"]
 
 
-class HipKernels(Products, Attention, Mixers, Hybrid):
+class HipKernels(Products, Attention, Mixers, Hybrid, Composite):
     def __init__(self, dtype=torch.bfloat16, device="cuda:0"):
         if dtype not in _DTYPE_CODE:
             raise ValueError(f"compute dtype must be float32 or bfloat16, not {dtype}")

@@ -276,7 +276,9 @@ class Attention:
         (float: scores become softcap * tanh(scores / softcap)), ``sinks`` (float32 [Hq]: one
         more logit per head in the softmax's sum, with no value) and ``slopes`` (float32 [Hq]:
         slope * (key position - query position) added to the scaled scores) and ``keep_first``
-        (int, with a window: the keys at positions below it stay visible to every later token). Such a layer,
+        (int, with a window: the keys at positions below it stay visible to every later token) and ``pooled`` (the
+        cache slot, whose pages of means hold one mean key and value per block of ``slot.pool`` positions: a token sees
+        the blocks that lie wholly before its window, in the same softmax). Such a layer,
         and one whose scale is not positive, goes to the kernel that computes scores on the
         vector units, in either dtype; the MFMA kernels take plain scores only."""
         N, Hq, D = q.shape
@@ -291,9 +293,9 @@ class Attention:
         out = torch.empty((N, Hq * D), dtype=self.dtype, device=self.device)
         w = int(window) if window else 0
         G = Hq // Hkv
-        softcap, sinks, slopes, keep_first = 0.0, None, None, 0
+        softcap, sinks, slopes, keep_first, means, pool = 0.0, None, None, 0, None, 0
         if terms:
-            known = {"softcap", "sinks", "slopes", "keep_first", "zero_sink"}
+            known = {"softcap", "sinks", "slopes", "keep_first", "zero_sink", "pooled"}
             if set(terms) - known:
                 raise KernelError(f"attention: unknown score terms {sorted(set(terms) - known)}")
             softcap = float(terms.get("softcap") or 0.0)
@@ -306,14 +308,23 @@ class Attention:
             for name, t in (("sinks", sinks), ("slopes", slopes)):
                 if t is not None:
                     self._want(t, name, torch.float32, (Hq,))
-        plain = softcap == 0.0 and sinks is None and slopes is None and scale > 0 and keep_first == 0
+            if terms.get("pooled") is not None:
+                # the slot itself: its pages of means and how many positions a mean stands for
+                means, pool = terms["pooled"].pooled, int(terms["pooled"].pool)
+                if means is None or pool < 1 or not w or keep_first or slopes is not None:
+                    raise KernelError("attention: pooled blocks need a window, the slot's pages of means, and neither kept "
+                                      "first keys nor a bias by distance")
+                self._check_slot(means, Hkv, D)
+                if means.block_size != slot.block_size:
+                    raise KernelError("attention: the pages of means hold as many entries as the tokens' pages")
+        plain = softcap == 0.0 and sinks is None and slopes is None and scale > 0 and keep_first == 0 and not pool
         # The kernel that shares K and V tiles among four waves also takes kept first keys and an added weight of
         # score 0 (``sinks`` all zero: ``terms["zero_sink"]`` says so without a look at the device); the per-wave
         # kernel with key splits does not, so a step with a long portion sends all its rows to the former (behind
         # a window no row walks far), and steps of short portions and decoded tokens go to the vector-unit kernel.
         zero_sink = bool(terms and terms.get("zero_sink")) and sinks is not None
         windowed = (softcap == 0.0 and slopes is None and scale > 0 and (sinks is None or zero_sink)
-                    and (keep_first > 0 or zero_sink))
+                    and (keep_first > 0 or zero_sink) and not pool)
         if self.dtype == torch.bfloat16 and self.attention_mfma and (plain or windowed):
             gpl = max(0, (min(G, 16) - 1).bit_length())
             decode = getattr(ctx, "max_q_len", 1) == 1
@@ -387,6 +398,8 @@ class Attention:
                 return out
         self.last_attention_kernel = ("tokens", 0)
         max_keys = ctx.max_ctx_len if not w else min(w + keep_first, ctx.max_ctx_len)
+        if pool:
+            max_keys = min(w, ctx.max_ctx_len) + max(0, ctx.max_ctx_len - w) // pool
         split_len, n_splits = self.plan_splits(N, Hkv, G, max_keys)
         part_o = part_ml = None
         if n_splits > 1:
@@ -403,5 +416,7 @@ class Attention:
                 _ptr(part_ml[lo:lo + n]) if part_ml is not None else None,
                 c_int(n), c_int(Hq), c_int(Hkv), c_int(slot.block_size), c_float(scale), c_int(w),
                 c_int(split_len), c_int(n_splits), c_int(self.code), c_float(softcap), _ptr(sinks), _ptr(slopes),
-                c_int(keep_first), self._stream()), "paged_attention")
+                c_int(keep_first), _ptr(means.k if pool else None), _ptr(means.v if pool else None),
+                _ptr(means.block_table if pool else None), c_int(means.block_table.shape[1] if pool else 0), c_int(pool),
+                self._stream()), "paged_attention")
         return out

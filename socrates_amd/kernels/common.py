@@ -59,7 +59,7 @@ _MIXER_SIGNATURES = {
     "soc_wkv": [P, P, P, P, P, I, I, P, L, I, P, P, P, I, I, I, P],
     "soc_causal_conv_silu": [P, I, I, I, P, P, I, P, L, I, P, P, P, I, I, I, P],
     "soc_ssd": [P, P, P, P, P, I, I, I, I, P, L, I, P, P, P, I, I, I, P],
-    "soc_gated_group_norm": [P, P, I, P, I, I, I, F, I, P, I, P],
+    "soc_gated_group_norm": [P, P, I, P, I, I, I, F, I, I, P, I, P],
     "soc_latent_write": [P, I, I, I, I, P, F, P, I, P, P, P, I, P, I, I, I, P],
     "soc_rmsnorm_cols": [P, I, P, P, I, I, F, I, P],
     "soc_latent_query_turn": [P, I, I, I, I, I, I, P, I, P, P, I, P],
@@ -77,9 +77,20 @@ _HYBRID_SIGNATURES = {
     "soc_side_gate": [P, P, I, I, P, I, P, I, I, I, P],
     "soc_add_cast": [P, P, P, I, L, P, I, P],
 }
+_COMPOSITE_SIGNATURES = {
+    "soc_norm_add_cast": [P, P, I, P, F, P, I, I, I, P],
+    "soc_depth_begin": [P, P, P, L, I, P],
+    "soc_depth_average": [P, P, I, P, P, L, I, P],
+    "soc_window_prepare": [P, I, I, I, I, P, P, P, P, P, I, P, P, P, P, I, F, P, I, P, I, I, I, I, I, I, I, I, P],
+    "soc_pool_blocks": [P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
+    "soc_turn_back": [P, P, P, P, I, I, I, I, I, P],
+    "soc_linear_attention": [P, I, I, I, I, F, I, P, P, P, F, I, I, I, P, L, I, P, P, P, I, I, I, P],
+    "soc_scaled_sum": [P, I, F, P, I, F, P, P, I, I, I, P],
+    "soc_glu_gelu": [P, P, I, I, I, I, P],
+}
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {
-    "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, F, P, P, I, P],
+    "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, F, P, P, I, P, P, P, I, I, P],
     "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, P],
     "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, I, I, P],
     "soc_paged_attention_decode_fused": [P, I, P, P, P, I, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P, P, P, F, I, I, P],

@@ -159,9 +159,10 @@ class Mixers:
                                       _ptr(out), c_int(ctx.n_seqs), c_int(ctx.max_q_len), c_int(self.code), self._stream()), "ssd")
         return out
 
-    def gated_group_norm(self, y, z, gain, groups, eps, gate_first=True):
+    def gated_group_norm(self, y, z, gain, groups, eps, gate_first=True, sigmoid=False):
         """y (float32 [N, inner]) * silu(z[:, :inner]), RMS-normed in ``groups`` equal parts, times gain;
-        ``gate_first`` False: y normed, times gain, and only then times silu(z)."""
+        ``gate_first`` False: y normed, times gain, and only then times silu(z). ``sigmoid``: the gate is
+        sigmoid(z) in place of silu(z)."""
         N, inner = y.shape
         self._want(y, "y", torch.float32)
         self._want(z, "z", self.dtype)
@@ -170,7 +171,8 @@ class Mixers:
             raise KernelError(f"gated norm: z {tuple(z.shape)} against y {tuple(y.shape)} in {groups} parts")
         out = torch.empty((N, inner), dtype=self.dtype, device=self.device)
         _check(self._mixers().soc_gated_group_norm(_ptr(y), _ptr(z), c_int(z.shape[1]), _ptr(gain), c_int(N), c_int(inner),
-                                                   c_int(groups), c_float(eps), c_int(1 if gate_first else 0), _ptr(out),
+                                                   c_int(groups), c_float(eps), c_int(1 if gate_first else 0), c_int(1 if sigmoid else 0),
+                                                   _ptr(out),
                                                    c_int(self.code), self._stream()),
                "gated_group_norm")
         return out

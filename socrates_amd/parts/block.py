@@ -264,10 +264,16 @@ class DepthAverageBlock:
         depth = self.depth.spec
         # the stream in the compute dtype, for the mixer: the block before has left it, or it is cast here
         # (with whatever that block left un-added)
-        x = pending.rows if isinstance(pending, Normed) else ops.add_cast(residual, pending)
+        if isinstance(pending, Normed):
+            x = pending.rows
+        elif pending is not None or depth.index != 0:
+            x = ops.add_cast(residual, pending)
         if depth.index == 0:
             # the first layer of a step files the embedding output as X_0
-            ctx.carry[self._CARRY] = ops.depth_begin(residual, depth.n_layers + 1)
+            if pending is None:
+                ctx.carry[self._CARRY], x = ops.depth_begin(residual, depth.n_layers + 1, cast=True)
+            else:
+                ctx.carry[self._CARRY] = ops.depth_begin(residual, depth.n_layers + 1)
         kept = ctx.carry[self._CARRY]
         gain, eps = self.post1.fusable()
         x = ops.norm_add_cast(residual, self.mixer.forward(x, ctx, slot, write), gain, eps, cast=self.ffn is not None)

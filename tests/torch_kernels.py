@@ -426,10 +426,10 @@ class TorchKernels:
         return residual.to(self.dtype)
 
     # -- norms on results with a weighted sum over depth; window attention with pooled blocks; linear attention ----
-    def depth_begin(self, residual, total):
+    def depth_begin(self, residual, total, cast=False):
         kept = torch.zeros((total,) + tuple(residual.shape), dtype=residual.dtype, device=residual.device)
         kept[0] = residual
-        return kept
+        return (kept, residual.to(self.dtype)) if cast else kept
 
     def norm_add_cast(self, residual, y, gain, eps, cast=True):
         residual += self._norm(y, gain, eps).to(residual.dtype)
