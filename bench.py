@@ -367,6 +367,75 @@ def tedulorn_beside_others(args, dtype, item):
     return 0
 
 
+def pozalorn_dict(width, ff, n_layers, heads, kv_heads, window=1024, pool=64):
+    """A Pozalorn of ``n_layers`` layers at a real model's layer sizes, four kinds in turn: windowed attention with a
+    sink per head beside lightning attention (heads of 128 x 128), two layers of gated linear attention (a state of
+    128 x 256 per head, decay logits through a rank of 16), and windowed attention with q and k normed whole,
+    values turned by position and one mean key and value per ``pool`` tokens before the window; every feed-forward
+    gated and dense; the stream after a layer a weighted sum over depth."""
+    rot = {"base": 1000000.0, "dims": 128, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "rot": rot, "mask": {"size": window}}
+    n_lin = width // 128
+    right = {"heads": n_lin, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** (-5 - 4 * h / n_lin) for h in range(n_lin)]}
+    gla = {"type": "gla", "mixer": {"heads": width // 256, "dim": 128, "vdim": 256, "tau": 16.0}}
+    pooled = dict(left, mask={"size": window, "pool": pool})
+    kinds = [{"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.7, "right_scale": 0.7}}, gla, gla,
+             {"type": "attention", "mixer": pooled}]
+    layers = []
+    for i in range(n_layers):
+        layer = json.loads(json.dumps(kinds[i % 4]))
+        layer["mlp"] = {"kind": "dense", "ff": ff}
+        layers.append(layer)
+    return {"architecture": "Pozalorn", "vocab": 151936, "width": width, "layers": layers, "norm": {"eps": 1e-6}}
+
+
+def pozalorn_beside_others(args, dtype, item):
+    """Prefill and decode of Pozalorn at a few real layer sizes, beside Tedulorn (the closest model: windowed attention
+    and a linear recurrence in turn) and Qwen3 of the same width, feed-forward size, vocabulary and number of layers,
+    all with the library's default solutions for its products. One JSON line of its own; the default workload and
+    its line are untouched."""
+    import torch
+    sizes = [("4b", "qwen3-4b"), ("8b", "qwen3-8b")]
+    n_layers = args.layers or 12
+    out = {"metric": "prefill and decode of Pozalorn beside Tedulorn and Qwen3 at equal width, feed-forward, vocabulary and layers",
+           "dtype": args.dtype, "layers": n_layers, "batch": args.batch, "context": args.context,
+           "prefill_tokens": args.prefill_tokens, "data": "synthetic: seeded random weights, uniform random token ids",
+           "sizes": {}}
+    only = set(filter(None, (args.only or "").split(",")))
+    for tag, preset in sizes:
+        if only & {name for name, _ in sizes} and tag not in only:
+            continue
+        q = preset_dict(preset)
+        q["num_hidden_layers"] = n_layers
+        t = tedulorn_dict(q["hidden_size"], q["intermediate_size"], n_layers, q["num_attention_heads"], q["num_key_value_heads"])
+        p = pozalorn_dict(q["hidden_size"], q["intermediate_size"], n_layers, q["num_attention_heads"], q["num_key_value_heads"])
+        point = {}
+        for name, cfg in (("pozalorn", p), ("tedulorn", t), ("qwen3", q)):
+            if only & {"pozalorn", "tedulorn", "qwen3"} and name not in only:
+                continue
+            config, engine = build_engine(cfg, dtype, args.batch, args.max_len, seed=0, compile_=not args.no_graphs,
+                                          chunk=max(2048, args.prefill_tokens), block_size=args.block_size)
+            V = cfg.get("vocab_size") or cfg["vocab"]
+            tok_s, ms = decode_rate(engine, args.batch, args.context, args.steps, args.warmup, V, seed=1)
+            pre_s = prefill_rate(engine, args.prefill_tokens, V, seed=2)
+            if name == "qwen3":
+                weights = config.param_counts()["read_per_step"] * item
+                cache = args.batch * args.context * config.kv_bytes_per_token(item)
+            else:
+                weights = config.step_weight_bytes(args.batch, item)
+                cache = config.step_cache_bytes(args.batch, args.context, item)
+            point[name] = {"decode_tok_s": round(tok_s, 1), "decode_ms": round(ms, 4),
+                           "decode_hbm_frac": round((weights + cache) / (ms * 1e-3) / 1e9 / HBM_GBPS, 4),
+                           "prefill_ms": round(pre_s * 1e3, 3), "prefill_tok_s": round(args.prefill_tokens / pre_s, 1),
+                           "prefill_flop_frac": round(config.prefill_flops(args.prefill_tokens) / pre_s / PEAK_FLOPS[args.dtype], 4),
+                           "weights_gb": round(weights / 1e9, 3)}
+            release(engine)
+            torch.cuda.synchronize()
+        out["sizes"][tag] = point
+    print(json.dumps(out))
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -389,7 +458,11 @@ def main(argv=None):
     ap.add_argument("--tedulorn", action="store_true",
                     help="instead of the default workload: prefill and decode of Tedulorn at 4B- and 8B-sized layers "
                          "(--layers of them, default 12), each beside Mitisun and Qwen3 of the same sizes")
-    ap.add_argument("--only", default=None, help="--tedulorn: sizes and models to run, with commas (4b,8b,tedulorn,mitisun,qwen3)")
+    ap.add_argument("--pozalorn", action="store_true",
+                    help="instead of the default workload: prefill and decode of Pozalorn at 4B- and 8B-sized layers "
+                         "(--layers of them, default 12), each beside Tedulorn and Qwen3 of the same sizes")
+    ap.add_argument("--only", default=None,
+                    help="--tedulorn, --pozalorn: sizes and models to run, with commas (4b,8b,pozalorn,tedulorn,mitisun,qwen3)")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per page of the cache (the reference's 16)")
     ap.add_argument("--no-graphs", action="store_true")
@@ -421,6 +494,8 @@ def main(argv=None):
         return mitisun_beside_qwen3(args, dtype, item)
     if args.tedulorn:
         return tedulorn_beside_others(args, dtype, item)
+    if args.pozalorn:
+        return pozalorn_beside_others(args, dtype, item)
     if args.mixed:
         args.preset = args.preset or MIXED_PRESET
         args.max_len = max(args.max_len, 8192)

@@ -52,10 +52,11 @@ class StateSlot:
 class PagedGroup:
     """Cache slots with the same need: one allocator, one table, a pool pair per slot."""
 
-    def __init__(self, need: PagedKV, max_rows, table_width, block_size, num_blocks, dtype, device, per=1):
-        """``per``: positions that one entry of a page stands for (1: a token; P: the mean of a block of P
+    def __init__(self, need: PagedKV, max_rows, table_width, block_size, num_blocks, dtype, device, per=0):
+        """``per``: positions that one entry of a page stands for (0: a token; P >= 1: the mean of a block of P
         tokens, which exists once the block is complete and is never given back before the row closes)."""
-        self.need, self.block_size, self.table_width, self.per = need, block_size, table_width, per
+        self.need, self.block_size, self.table_width = need, block_size, table_width
+        self.means, self.per = per > 0, max(per, 1)
         self.allocator = BlockAllocator(num_blocks)
         # one row more than can be opened: the null row, whose entries all point at the null
         # page, stands in for the padding rows of a fixed-width (captured) decode step
@@ -66,7 +67,7 @@ class PagedGroup:
         self.first_live = [0] * max_rows
         # with a window that keeps the first positions visible: the blocks that hold them stay with the
         # row whatever the window has passed (a row then holds blocks 0 .. kept and first_live .. covered)
-        keep_first = getattr(need, "keep_first", 0) if need.window is not None and per == 1 else 0
+        keep_first = getattr(need, "keep_first", 0) if need.window is not None and not self.means else 0
         self.kept_blocks = blocks_for(keep_first, block_size) if keep_first > 0 else 0
         self.dirty = set()
         # a latent is kept as one "head" of ``width`` elements, in one pool per slot
@@ -85,7 +86,7 @@ class PagedGroup:
     # -- pages a row needs / can drop ---------------------------------------------------------
     def droppable(self, row: int, next_start: int) -> int:
         """Logical blocks of ``row`` that no token at position >= next_start can see."""
-        if self.need.window is None or self.per > 1:
+        if self.need.window is None or self.means:
             return self.first_live[row]
         first_visible = max(0, next_start - self.need.window + 1)
         pool = getattr(self.need, "pool", 0)
@@ -199,10 +200,10 @@ class CacheManager:
         self.scalars = RowScalars(max_rows)
         self._open = [False] * max_rows
 
-    def _group(self, key, need, num_blocks, per=1):
+    def _group(self, key, need, num_blocks, per=0):
         group = self._by_need.get(key)
         if group is None:
-            table_width = self.table_width if per == 1 else blocks_for(self.max_len // per, self.block_size)
+            table_width = self.table_width if not per else blocks_for(self.max_len // per, self.block_size)
             group = PagedGroup(need, self.max_rows, max(table_width, 1), self.block_size, num_blocks, self.dtype,
                                self.device, per=per)
             self._by_need[key] = group
@@ -225,10 +226,10 @@ class CacheManager:
             k, v = group.pools[serial]
             slot = PagedSlot(k, v, group.table, self.block_size, need.window)
             if pool:
-                # the means of the blocks: as many entries as the tokens' pages hold blocks, and a page more per
-                # row for the rounding
-                entries = self._num_blocks * self.block_size // pool
-                means = self._group(("means", need), need, blocks_for(entries, self.block_size) + self.max_rows, per=pool)
+                # the means of the blocks stay with a row however far its window has moved on, so every row can
+                # hold those of max_len tokens (a pool-th of what the tokens themselves would take)
+                per_row = max(1, blocks_for(self.max_len // pool, self.block_size))
+                means = self._group(("means", need), need, self.max_rows * per_row, per=pool)
                 means.add_slot(serial)
                 mk, mv = means.pools[serial]
                 slot.pooled, slot.pool = PagedSlot(mk, mv, means.table, self.block_size, None), pool
