@@ -1123,6 +1123,10 @@ __device__ __forceinline__ int pf_k_row32(int k) { return (k & ~12) | ((k & 4) <
 
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 
+// Entry e of a row's pages of means walks through the prompt kernel as the key PF_MEAN + e (a multiple of every
+// page size, so a key's place in its page is the entry's).
+constexpr int PF_MEAN = -(1 << 30);
+
 // PAIR: pages hold an even, power-of-two number of keys, so a thread's two keys share a page.
 // M32: a wave owns 32 rows and multiplies with the 32 x 32 x 16 instruction (RT = 1; head
 // sizes that are multiples of 32): per row, half the loads, LDS reads, stores and barriers
@@ -1139,7 +1143,9 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                           int table_width, const int* __restrict__ token_rows,
                           const int* __restrict__ positions, const int* __restrict__ row_blocks,
                           bf16* __restrict__ out, int Hq, int Hkv, int BS, int bs_shift, float scale,
-                          int window, int group_pad_log2, int keep_first, int sink) {
+                          int window, int group_pad_log2, int keep_first, int sink, const float* __restrict__ sinks,
+                          const bf16* __restrict__ mean_k, const bf16* __restrict__ mean_v,
+                          const int* __restrict__ mean_table, int mean_table_width, int pool) {
     static_assert(D <= 128, "one key pair per thread");
     static_assert(KS == 1 || (KS == 2 && M32), "key halves come with the 32-row products");
     constexpr int PF_TILE_ELEMS = PF_K_ELEMS + PF_V_ELEMS;          // one K tile and one V^T tile
@@ -1168,9 +1174,18 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     // such tiles would reach into the window's, the walk starts at key 0 instead and the mask does the rest.
     int kept = window > 0 ? min(keep_first, kmin) : 0, n_pre = (kept + PF_KEYS - 1) / PF_KEYS;
     if (n_pre * PF_KEYS > (kmin & ~(PF_KEYS - 1))) { kmin = 0; kept = 0; n_pre = 0; }
+    // With pooled blocks (pool > 0, a window, no kept keys) the tiles in front of the window's hold the means of the
+    // blocks of pool positions that lie wholly before a row's window, from pages of their own: entry e of the row's
+    // pages of means is walked as the key PF_MEAN + e (negative, so a tile of means is known by its first key), and
+    // the row at position p sees the entries below (p - window + 1) / pool.
+    auto blocks_before = [&](int pos) { const int d = pos - window + 1; return d > 0 ? d / pool : 0; };
+    const int n_means = pool > 0 ? blocks_before(khi - 1) : 0;      // entries any row of the block sees
+    if (pool > 0) n_pre = (n_means + PF_KEYS - 1) / PF_KEYS;
+    const int* mtable = pool > 0 ? mean_table + (size_t)token_rows[tok0] * mean_table_width : table;
     int klo = kmin & ~(PF_KEYS - 1);
     const int first_real = klo;                                     // virtual keys from here on are real ones
     const int pre_shift = klo - n_pre * PF_KEYS;                    // a virtual key before that is the real key minus this
+    const int pre_base = (pool > 0 ? PF_MEAN : 0) - pre_shift;      // (or the entry of the pages of means, as PF_MEAN + entry)
     if (KS == 1) klo = pre_shift;
     // kend: where this half's walk over the tiles ends. Both halves take the same number of
     // steps (they share the barriers); the second may run past khi, where keys are stand-ins
@@ -1187,8 +1202,11 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     const int wave_hi_pos = min(khi, wave_lo_pos + tokens_per_wave) - 1;
     const bool wave_has_rows = wtok0 < ntok;
     const float c2 = scale * 1.44269504088896340736f;               // to base 2
+    const int means_lo = pool > 0 ? blocks_before(wave_lo_pos) : 0; // entries that all / any of the wave's rows see
+    const int means_hi = pool > 0 ? blocks_before(wave_hi_pos) : 0;
 
-    int row_pos[RT];
+    int row_pos[RT], mean_end[RT];                                  // (mean_end: the first entry of means a row does not see)
+    float sink_l2[RT];                                              // a learned sink (sink == 2), to base 2
     size_t row_q[RT];
     uint4 qf[RT][QK_STEPS];
 #pragma unroll
@@ -1198,6 +1216,8 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         const bool ok = tt < ntok && g < G;
         row_pos[rt] = ok ? pos0 + tt : -1;
         row_q[rt] = ((size_t)(tok0 + (ok ? tt : 0)) * Hq + (size_t)kvh * G + (ok ? g : 0)) * D;
+        mean_end[rt] = PF_MEAN + (pool > 0 && ok ? blocks_before(pos0 + tt) : 0);
+        sink_l2[rt] = sink == 2 && ok ? sinks[kvh * G + g] * 1.44269504088896340736f : 0.f;
 #pragma unroll
         for (int kk = 0; kk < QK_STEPS; ++kk)
             qf[rt][kk] = ok ? load_qk_slice(q + row_q[rt], kk, kb) : make_uint4(0u, 0u, 0u, 0u);
@@ -1213,7 +1233,8 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     // 32-row products: the lane's row is lane % 32, its half of every 16-wide k step lane / 32
     constexpr int DQ32 = D / 16, DB32 = D / 32;
     const int c32 = lane % 32, g32 = lane / 32;
-    int row_pos32 = -1;
+    int row_pos32 = -1, mean_end32 = PF_MEAN;
+    float sink32_l2 = 0.f;
     size_t row_q32 = 0;
     uint4 qf32[M32 ? DQ32 : 1];                           // the lane's slices of its query row
     f32x16_t o32[M32 ? DB32 : 1];
@@ -1223,6 +1244,8 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         const bool ok = tt < ntok && gh < G;
         row_pos32 = ok ? pos0 + tt : -1;
         row_q32 = ((size_t)(tok0 + (ok ? tt : 0)) * Hq + (size_t)kvh * G + (ok ? gh : 0)) * D;
+        if (pool > 0 && ok) mean_end32 = PF_MEAN + blocks_before(pos0 + tt);
+        if (sink == 2 && ok) sink32_l2 = sinks[kvh * G + gh] * 1.44269504088896340736f;
 #pragma unroll
         for (int t = 0; t < DQ32; ++t)
             qf32[t] = ok ? *reinterpret_cast<const uint4*>(q + row_q32 + 16 * t + 8 * g32) : make_uint4(0u, 0u, 0u, 0u);
@@ -1246,42 +1269,55 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     const size_t page_stride = (size_t)Hkv * BS * D;
     const bf16* k_base = k_pool + (size_t)kvh * BS * D + part_ld * 8;
     const bf16* v_base = v_pool + (size_t)kvh * BS * D + part_ld * 8;
+    // (the pools of means as distances from the tokens' pools, in elements: two scalars instead of two more pointers per thread)
+    const ptrdiff_t mk_off = pool > 0 ? mean_k - k_pool : 0, mv_off = pool > 0 ? mean_v - v_pool : 0;
     auto lookup = [&](int key0, int (&pg)[2]) {
+        const bool of_means = key0 < 0;                      // uniform: a tile of means, entries of the row's other table
+        const int* tb = of_means ? mtable : table;
+        if (of_means) key0 -= PF_MEAN;
         if constexpr (PAIR) {
             const int key = key0 + 2 * kp;
-            const bool ok = (key + 1 >= kmin || key < kept) && key < khi;
-            pg[0] = pg[1] = table[ok ? key >> bs_shift : 0];
+            const bool ok = of_means ? key < n_means : (key + 1 >= kmin || key < kept) && key < khi;
+            pg[0] = pg[1] = tb[ok ? key >> bs_shift : 0];
         } else {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int key = key0 + 2 * kp + h;
-                const bool ok = (key >= kmin || key < kept) && key < khi;
-                pg[h] = table[ok ? (bs_shift >= 0 ? key >> bs_shift : key / BS) : 0];
+                const bool ok = of_means ? key < n_means : (key >= kmin || key < kept) && key < khi;
+                pg[h] = tb[ok ? (bs_shift >= 0 ? key >> bs_shift : key / BS) : 0];
             }
         }
     };
     auto fetch = [&](int key0, const int (&pg)[2], uint4 (&kr)[2], uint4 (&vr)[2]) {
+        const bool of_means = key0 < 0;                      // uniform
+        const bf16* kb_ = k_base + (of_means ? mk_off : 0);
+        const bf16* vb_ = v_base + (of_means ? mv_off : 0);
+        if (of_means) key0 -= PF_MEAN;
         if constexpr (PAIR) {
             const size_t off = (size_t)pg[0] * page_stride + (size_t)(((key0 + 2 * kp) & (BS - 1)) * D);
-            kr[0] = *reinterpret_cast<const uint4*>(k_base + off);
-            kr[1] = *reinterpret_cast<const uint4*>(k_base + off + D);
-            vr[0] = *reinterpret_cast<const uint4*>(v_base + off);
-            vr[1] = *reinterpret_cast<const uint4*>(v_base + off + D);
+            kr[0] = *reinterpret_cast<const uint4*>(kb_ + off);
+            kr[1] = *reinterpret_cast<const uint4*>(kb_ + off + D);
+            vr[0] = *reinterpret_cast<const uint4*>(vb_ + off);
+            vr[1] = *reinterpret_cast<const uint4*>(vb_ + off + D);
         } else {
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int key = key0 + 2 * kp + h;
                 const int in_page = bs_shift >= 0 ? key & (BS - 1) : key % BS;
                 const size_t off = (size_t)pg[h] * page_stride + (size_t)(in_page * D);
-                kr[h] = *reinterpret_cast<const uint4*>(k_base + off);
-                vr[h] = *reinterpret_cast<const uint4*>(v_base + off);
+                kr[h] = *reinterpret_cast<const uint4*>(kb_ + off);
+                vr[h] = *reinterpret_cast<const uint4*>(vb_ + off);
             }
         }
     };
     auto stash = [&](int buf, int key0, const uint4 (&kr)[2], const uint4 (&vr)[2]) {
         if (!loader) return;
         uint4 k0 = kr[0], k1 = kr[1], v0 = vr[0], v1 = vr[1];
-        if (key0 < kmin || key0 + PF_KEYS > khi) {           // uniform: a tile at an edge of the range
+        if (key0 < 0) {                                      // uniform: a tile of means, past the last one that is seen
+            const int e = key0 - PF_MEAN + 2 * kp;
+            if (e >= n_means) { k0 = make_uint4(0u, 0u, 0u, 0u); v0 = k0; }
+            if (e + 1 >= n_means) { k1 = make_uint4(0u, 0u, 0u, 0u); v1 = k1; }
+        } else if (key0 < kmin || key0 + PF_KEYS > khi) {    // uniform: a tile at an edge of the range
             const int key = key0 + 2 * kp;
             if ((key < kmin && key >= kept) || key >= khi) { k0 = make_uint4(0u, 0u, 0u, 0u); v0 = k0; }
             if ((key + 1 < kmin && key + 1 >= kept) || key + 1 >= khi) { k1 = make_uint4(0u, 0u, 0u, 0u); v1 = k1; }
@@ -1332,6 +1368,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                     const int key = key0 + 8 * kb + r;
                     bool seen = key <= row_pos[rt];
                     if (window > 0) seen = seen && (key > row_pos[rt] - window || key < keep_first);
+                    if (key0 < 0) seen = key < mean_end[rt];          // (uniform: a tile of means)
                     t[r] = seen ? t[r] : -INFINITY;
                 }
                 mx = fmaxf(mx, t[r]);
@@ -1398,6 +1435,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                 const int key = key0 + 16 * (i / 8) + 8 * g32 + i % 8;
                 bool seen = key <= row_pos32;
                 if (window > 0) seen = seen && (key > row_pos32 - window || key < keep_first);
+                if (key0 < 0) seen = key < mean_end32;               // (uniform: a tile of means)
                 sc[i] = seen ? sc[i] : -INFINITY;
             }
             mx = fmaxf(mx, sc[i]);
@@ -1462,11 +1500,12 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     // not: the main loop takes the rounds in which both buffers have a tile to load, and
     // the last tiles (at most three) follow without a loop.
     auto tile = [&](int key0, int buf) {
-        if (wave_has_rows && key0 <= wave_hi_pos) {
+        const bool of_means = key0 < 0;                      // uniform
+        if (wave_has_rows && (of_means ? key0 - PF_MEAN < means_hi : key0 <= wave_hi_pos)) {
             // whole: every key of the tile is at or before the wave's first position and inside
-            // the window of its last one
-            const bool whole = key0 + PF_KEYS - 1 <= wave_lo_pos &&
-                               (window <= 0 || key0 > wave_hi_pos - window);
+            // the window of its last one (of means: all its entries are seen by the wave's first row)
+            const bool whole = of_means ? key0 - PF_MEAN + PF_KEYS <= means_lo
+                                        : key0 + PF_KEYS - 1 <= wave_lo_pos && (window <= 0 || key0 > wave_hi_pos - window);
             if constexpr (M32) {
                 uint4 pf[2];
                 float alpha;
@@ -1487,7 +1526,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     int pg0[2], pg1[2];
     uint4 kr0[2], vr0[2], kr1[2], vr1[2];
     // (the walk is over virtual keys: the tiles of the kept first keys stand in front of the window's)
-    auto real = [&](int v) { return v < first_real ? v - pre_shift : v; };
+    auto real = [&](int v) { return v < first_real ? v + pre_base : v; };
     lookup(real(klo), pg0);
     lookup(real(klo + PF_KEYS), pg1);
     fetch(real(klo), pg0, kr0, vr0);
@@ -1551,7 +1590,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 #pragma unroll
                 for (int i = 0; i < 16; ++i) o32[b][i] = o32[b][i] * wa + xch[(16 * b + i) * 64] * wb;
         }
-        if (sink) L += __builtin_amdgcn_exp2f(-m_ref);       // one more weight of score 0, no value
+        if (sink) L += __builtin_amdgcn_exp2f(sink32_l2 - m_ref);   // one more weight (of score 0, or the head's own), no value
         if (row_pos32 >= 0) {
             const float inv = L > 0.f ? 1.0f / L : 0.f;
 #pragma unroll
@@ -1571,7 +1610,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         float L = l[rt];
         L = sum_xor32(sum_xor16(L));
         if (row_pos[rt] < 0) continue;
-        if (sink) L += __builtin_amdgcn_exp2f(-(m[rt] == -INFINITY ? 0.f : m[rt]));   // one more weight of score 0, no value
+        if (sink) L += __builtin_amdgcn_exp2f(sink_l2[rt] - (m[rt] == -INFINITY ? 0.f : m[rt]));   // one more weight, no value
         const float inv = L > 0.f ? 1.0f / L : 0.f;
 #pragma unroll
         for (int j = 0; j < DV; ++j) {
@@ -1588,17 +1627,23 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 // one sequence, or null: every token is a block of its own. row_tiles 32: a wave owns 32 rows
 // (blocks of at most 4 * (32 >> group_pad_log2) tokens), head sizes that are multiples of 32;
 // row_tiles 64: the same with eight waves, four for each half of a block's keys. keep_first (with a window): the
-// keys below it stay visible to every row (not with row_tiles 64); sink: one more weight of score 0 and no value
-// in every row's sum.
+// keys below it stay visible to every row (not with row_tiles 64); sink 1: one more weight of score 0 and no value
+// in every row's sum; sink 2: of the score sinks[head] (not scaled). pool > 0 (with a window, not with kept keys or
+// row_tiles 64): a row also sees the means of the blocks of pool positions that lie wholly before its window, entries
+// of the pools mean_k, mean_v (pages of BS entries, table mean_table).
 SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, const void* v_pool,
                                            const int* block_table, int table_width, const int* token_rows,
                                            const int* positions, const int* row_blocks, int n_row_blocks,
                                            void* out, int N, int Hq, int Hkv, int BS, float scale,
                                            int window, int row_tiles, int group_pad_log2, int keep_first, int sink,
-                                           hipStream_t stream) {
+                                           const float* sinks, const void* mean_k, const void* mean_v, const int* mean_table,
+                                           int mean_table_width, int pool, hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
     if (Hkv < 1 || Hq % Hkv || BS < 1 || keep_first < 0) return (int)hipErrorInvalidValue;
     if (row_tiles == 64 && (keep_first > 0 && window > 0)) return (int)hipErrorInvalidValue;   // no kept keys with key halves
+    if (sink < 0 || sink > 2 || (sink == 2 && !sinks)) return (int)hipErrorInvalidValue;
+    if (pool < 0 || (pool > 0 && (window <= 0 || keep_first > 0 || row_tiles == 64 || !mean_k || !mean_v || !mean_table)))
+        return (int)hipErrorInvalidValue;                        // no means with kept keys or key halves
     if (!(scale > 0.f)) return (int)hipErrorInvalidValue;        // the maximum is taken of the raw scores
     if (!row_blocks && n_row_blocks != N) return (int)hipErrorInvalidValue;
     const int G = Hq / Hkv;
@@ -1611,7 +1656,7 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
     if constexpr (D <= 128) {
 #define SOC_PF_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, bs_shift, scale, window, group_pad_log2, \
-        keep_first, sink
+        keep_first, sink, sinks, (const bf16*)mean_k, (const bf16*)mean_v, mean_table, mean_table_width, pool
         const bool pair = bs_shift >= 1;
 #define SOC_PF_LAUNCH(RT_, M32_, KS_)                                                                            \
     do {                                                                                                    \

@@ -30,11 +30,51 @@ norm_add_cast_kernel(float* __restrict__ residual, const Y* __restrict__ y, cons
     }
 }
 
+// The same for rows of up to 256 * 8 * C elements, a multiple of 8: a thread keeps its C runs of 8 in registers
+// between the sum of squares and the sum into the stream.
+template <typename T, typename Y, int C>
+__global__ void __launch_bounds__(256)
+norm_add_cast_vec8_kernel(float* __restrict__ residual, const Y* __restrict__ y, const float* __restrict__ gain, float eps,
+                          T* __restrict__ out, int d) {
+    __shared__ float scratch[16];
+    const size_t row = (size_t)blockIdx.x * d;
+    float v[C][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int at = (threadIdx.x + c * 256) * 8;
+        if (at < d) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { v[c][e] = to_float(y[row + at + e]); ss = fmaf(v[c][e], v[c][e], ss); }
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int at = (threadIdx.x + c * 256) * 8;
+        if (at < d) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float r = residual[row + at + e] + v[c][e] * inv * gain[at + e];
+                residual[row + at + e] = r;
+                if (out) out[row + at + e] = from_float<T>(r);
+            }
+        }
+    }
+}
+
 SOC_EXPORT int soc_norm_add_cast(float* residual, const void* y, int y_f32, const float* gain, float eps, void* out, int N,
                                  int d, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
     if (d < 1) return (int)hipErrorInvalidValue;
-#define SOC_NAC(T, Y) hipLaunchKernelGGL((norm_add_cast_kernel<T, Y>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d)
+#define SOC_NAC(T, Y)                                                                                                                \
+    do {                                                                                                                             \
+        if (d % 8 == 0 && d <= 2048) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 1>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d);      \
+        else if (d % 8 == 0 && d <= 4096) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 2>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d); \
+        else if (d % 8 == 0 && d <= 8192) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 4>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d); \
+        else hipLaunchKernelGGL((norm_add_cast_kernel<T, Y>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d);                                     \
+    } while (0)
     if (dtype == 0) SOC_NAC(float, float);
     else if (y_f32) SOC_NAC(bf16, float);
     else SOC_NAC(bf16, bf16);
@@ -97,7 +137,7 @@ SOC_EXPORT int soc_depth_average(float* residual, float* kept, int count, const 
 // [D]; 2: over the whole of q (gain [Hq D]) and the whole of k (gain [Hkv D]). Then elements 2i and 2i + 1 of the
 // first 2 * half of every q and k head are turned by position * inv_freq[i], and (value_freq given) elements 2m and
 // 2m + 1 of every v head by position * value_freq[m]. q goes to q_out [N, Hq, P], k and v to the token's place in the
-// pools [pages, Hkv, BS, P], zeros behind D and Dv. One workgroup per token; q and k pass through LDS (dynamic,
+// pools [pages, Hkv, BS, P] (P even), zeros behind D and Dv. One workgroup per token; q and k pass through LDS (dynamic,
 // (Hq + Hkv) D floats).
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -142,38 +182,32 @@ window_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int
     }
     const int page = table[(size_t)token_rows[n] * table_width + pos / BS];
     const size_t place = (size_t)page * Hkv * BS + (size_t)(pos % BS);
-    // q and k heads: turned pairs, padding
-    for (int e = tid; e < (Hq + Hkv) * P; e += 256) {
-        const int h = e / P, i = e % P;
-        float y = 0.f;
-        if (i < D) {
+    // A thread owns one pair (2j, 2j + 1) of the padded head size and walks heads with it: the pair's angle is taken
+    // once (P is even: the pools' head size; 256 / (P / 2) threads share a pair's heads among them).
+    const int PP = P / 2, lanes = 256 / PP;                // (P <= 256: at least two threads per pair)
+    const int j = tid % PP, g = tid / PP;
+    if (g < lanes) {
+        float sn = 0.f, cs = 1.f;
+        if (j < half) sincosf((float)pos * inv_freq[j], &sn, &cs);
+        for (int h = g; h < Hq + Hkv; h += lanes) {
             const float* head = qk + (size_t)h * D;
-            y = head[i];
-            if (i < 2 * half) {
-                float sn, cs;
-                sincosf((float)pos * inv_freq[i >> 1], &sn, &cs);
-                y = (i & 1) ? head[i] * cs + head[i - 1] * sn : head[i] * cs - head[i + 1] * sn;
-            }
+            const float a = 2 * j < D ? head[2 * j] : 0.f, b = 2 * j + 1 < D ? head[2 * j + 1] : 0.f;
+            const float y0 = j < half ? a * cs - b * sn : a, y1 = j < half ? b * cs + a * sn : b;
+            T* dst = h < Hq ? q_out + ((size_t)n * Hq + h) * P : k_pool + (place + (size_t)(h - Hq) * BS) * P;
+            dst[2 * j] = from_float<T>(y0);
+            dst[2 * j + 1] = from_float<T>(y1);
         }
-        if (h < Hq) q_out[((size_t)n * Hq + h) * P + i] = from_float<T>(y);
-        else k_pool[(place + (size_t)(h - Hq) * BS) * P + i] = from_float<T>(y);
-    }
-    // v heads
-    for (int e = tid; e < Hkv * P; e += 256) {
-        const int h = e / P, i = e % P;
-        float y = 0.f;
-        if (i < Dv) {
-            const int c = col_v + h * Dv + i;
-            y = to_float(row[c]) + (bias ? bias[c] : 0.f);
-            if (value_freq) {
-                const int cp = (i & 1) ? c - 1 : c + 1;
-                const float other = to_float(row[cp]) + (bias ? bias[cp] : 0.f);
-                float sn, cs;
-                sincosf((float)pos * value_freq[i >> 1], &sn, &cs);
-                y = (i & 1) ? y * cs + other * sn : y * cs - other * sn;
-            }
+        // v heads
+        sn = 0.f; cs = 1.f;
+        if (value_freq && 2 * j + 1 < Dv) sincosf((float)pos * value_freq[j], &sn, &cs);
+        for (int h = g; h < Hkv; h += lanes) {
+            const int c = col_v + h * Dv + 2 * j;
+            const float a = 2 * j < Dv ? to_float(row[c]) + (bias ? bias[c] : 0.f) : 0.f;
+            const float b = 2 * j + 1 < Dv ? to_float(row[c + 1]) + (bias ? bias[c + 1] : 0.f) : 0.f;
+            T* dst = v_pool + (place + (size_t)h * BS) * P;
+            dst[2 * j] = from_float<T>(a * cs - b * sn);
+            dst[2 * j + 1] = from_float<T>(b * cs + a * sn);
         }
-        v_pool[(place + (size_t)h * BS) * P + i] = from_float<T>(y);
     }
 }
 
@@ -183,7 +217,7 @@ SOC_EXPORT int soc_window_prepare(const void* x, int ld, int col_q, int col_k, i
                                   const float* inv_freq, int half, const float* value_freq, int N, int Hq, int Hkv, int D,
                                   int Dv, int P, int BS, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (D < 1 || Dv < 1 || D > P || Dv > P || P > 256 || 2 * half > D || BS < 1 || norm < 0 || norm > 2 || Hq < 1 || Hkv < 1)
+    if (D < 1 || Dv < 1 || D > P || Dv > P || P > 256 || P % 2 || 2 * half > D || BS < 1 || norm < 0 || norm > 2 || Hq < 1 || Hkv < 1)
         return (int)hipErrorInvalidValue;
     if (norm && (!q_gain || !k_gain)) return (int)hipErrorInvalidValue;
     if (half && !inv_freq) return (int)hipErrorInvalidValue;
@@ -284,6 +318,29 @@ SOC_EXPORT int soc_turn_back(const void* o, void* out, const int* positions, con
     return soc_last_error();
 }
 
+// q (activated if act, scaled), k (activated if act) and, with z, the decay exp(logsigmoid(z + z_bias) / tau) of every
+// token, head and key channel, float32: prep [N, 2 or 3, H * D]. Ahead of the walk over a long portion, where each of a
+// head's workgroups would otherwise take them again.
+template <typename T>
+__global__ void linear_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, float q_scale, int act,
+                                      const float* __restrict__ z, const float* __restrict__ z_bias, float inv_tau, int HD,
+                                      size_t total, float* __restrict__ prep) {
+    const int planes = z ? 3 : 2;
+    for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+        const int c = (int)(e % HD);
+        const size_t n = e / HD;
+        float a = to_float(x[n * ld + col_q + c]), b = to_float(x[n * ld + col_k + c]);
+        if (act) { a = cmp_silu(a); b = cmp_silu(b); }
+        float* row = prep + n * planes * HD + c;
+        row[0] = a * q_scale;
+        row[HD] = b;
+        if (z) {
+            const float u = z[n * HD + c] + z_bias[c];
+            row[2 * (size_t)HD] = expf((fminf(u, 0.f) - log1pf(expf(-fabsf(u)))) * inv_tau);
+        }
+    }
+}
+
 // ---- linear attention: S <- diag(decay) S + k v^T, o = S^T q ------------------------------------------------------
 // x: rows of ld elements with H heads of D (q, from col_q; k, from col_k) and H heads of Dv (v, from col_v); with
 // act they pass silu; q is scaled by q_scale. CHANNEL: the decay of token t, head h, key channel i is
@@ -295,7 +352,8 @@ __global__ void __launch_bounds__(256)
 linear_attention_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int col_v, float q_scale, int act,
                         const float* __restrict__ decays, const float* __restrict__ z, const float* __restrict__ z_bias,
                         float inv_tau, int H, int D, int Dv, float* __restrict__ state, size_t stride, int offset,
-                        const int* __restrict__ seq_qstart, const int* __restrict__ seq_rows, float* __restrict__ out) {
+                        const int* __restrict__ seq_qstart, const int* __restrict__ seq_rows, const float* __restrict__ prep,
+                        float* __restrict__ out) {
     constexpr int REC_TB = rec_batch(DK), PARTS = 256 / CW, KPT = DK / PARTS, STAGE = (REC_TB * DK + 255) / 256;
     __shared__ float sq[2][REC_TB][DK], sk[2][REC_TB][DK];
     __shared__ float sa[CHANNEL ? 2 : 1][CHANNEL ? REC_TB : 1][CHANNEL ? DK : 1];
@@ -320,7 +378,13 @@ linear_attention_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, i
             const int e = tid + q * 256, t = e / DK, i = e % DK;
             const bool in = t < REC_TB && n0 + t < hi && i < D;
             float a = 0.f, b = 0.f, c = 1.f;
-            if (in) {
+            if (in && prep) {                          // activated, scaled and the decay taken ahead of the walk
+                const size_t HD = (size_t)H * D;
+                const float* row = prep + (size_t)(n0 + t) * (CHANNEL ? 3 : 2) * HD + head * D + i;
+                a = row[0];
+                b = row[HD];
+                if (CHANNEL) c = row[2 * HD];
+            } else if (in) {
                 const T* row = x + (size_t)(n0 + t) * ld + head * D + i;
                 a = to_float(row[col_q]);
                 b = to_float(row[col_k]);
@@ -401,11 +465,11 @@ template <typename T, int DK>
 static void launch_linear_attention(const void* x, int ld, int col_q, int col_k, int col_v, float q_scale, int act,
                                     const float* decays, const float* z, const float* z_bias, float inv_tau, int H, int D, int Dv,
                                     float* state, long long stride, int offset, const int* seq_qstart, const int* seq_rows,
-                                    float* out, int n_seqs, int cw, hipStream_t stream) {
+                                    const float* prep, float* out, int n_seqs, int cw, hipStream_t stream) {
 #define SOC_LA_LAUNCH(CW, CH)                                                                                                  \
     hipLaunchKernelGGL((linear_attention_kernel<T, DK, CW, CH>), dim3(H * ((Dv + CW - 1) / CW), n_seqs), dim3(256), 0, stream, \
                        (const T*)x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state,        \
-                       (size_t)stride, offset, seq_qstart, seq_rows, out)
+                       (size_t)stride, offset, seq_qstart, seq_rows, prep, out)
     if (z) { if (cw == 16) SOC_LA_LAUNCH(16, true); else SOC_LA_LAUNCH(64, true); }
     else   { if (cw == 16) SOC_LA_LAUNCH(16, false); else SOC_LA_LAUNCH(64, false); }
 #undef SOC_LA_LAUNCH
@@ -414,14 +478,26 @@ static void launch_linear_attention(const void* x, int ld, int col_q, int col_k,
 SOC_EXPORT int soc_linear_attention(const void* x, int ld, int col_q, int col_k, int col_v, float q_scale, int act,
                                     const float* decays, const float* z, const float* z_bias, float tau, int H, int D, int Dv,
                                     float* state, long long stride, int offset, const int* seq_qstart, const int* seq_rows,
-                                    float* out, int n_seqs, int max_q_len, int dtype, hipStream_t stream) {
+                                    float* prep, int n_tokens, float* out, int n_seqs, int max_q_len, int dtype,
+                                    hipStream_t stream) {
     if (n_seqs <= 0 || H <= 0) return 0;
     if (D < 1 || D > 256 || Dv < 1 || n_seqs > 65535) return (int)hipErrorInvalidValue;
     if ((z == nullptr) == (decays == nullptr) || (z && (!z_bias || !(tau > 0.f)))) return (int)hipErrorInvalidValue;
     const int cw = columns_per_workgroup(H, Dv, n_seqs, max_q_len);
     const float inv_tau = z ? 1.f / tau : 0.f;
-#define SOC_LA_F32(DK) launch_linear_attention<float, DK>(x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, cw, stream)
-#define SOC_LA_BF16(DK) launch_linear_attention<bf16, DK>(x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, out, n_seqs, cw, stream)
+    if (prep) {                                            // scratch [n_tokens, 2 or 3, H * D]
+        if (n_tokens <= 0) return (int)hipErrorInvalidValue;
+        const size_t total = (size_t)n_tokens * H * D;
+        const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+        if (dtype == 0)
+            hipLaunchKernelGGL(linear_prepare_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)x, ld, col_q, col_k,
+                               q_scale, act, z, z_bias, inv_tau, H * D, total, prep);
+        else
+            hipLaunchKernelGGL(linear_prepare_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (const bf16*)x, ld, col_q, col_k,
+                               q_scale, act, z, z_bias, inv_tau, H * D, total, prep);
+    }
+#define SOC_LA_F32(DK) launch_linear_attention<float, DK>(x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, prep, out, n_seqs, cw, stream)
+#define SOC_LA_BF16(DK) launch_linear_attention<bf16, DK>(x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, prep, out, n_seqs, cw, stream)
     if (dtype == 0) { SOC_BY_STATE_SIZE(D, SOC_LA_F32) } else { SOC_BY_STATE_SIZE(D, SOC_LA_BF16) }
     return soc_last_error();
 }

@@ -318,13 +318,14 @@ class Attention:
                 if means.block_size != slot.block_size:
                     raise KernelError("attention: the pages of means hold as many entries as the tokens' pages")
         plain = softcap == 0.0 and sinks is None and slopes is None and scale > 0 and keep_first == 0 and not pool
-        # The kernel that shares K and V tiles among four waves also takes kept first keys and an added weight of
-        # score 0 (``sinks`` all zero: ``terms["zero_sink"]`` says so without a look at the device); the per-wave
-        # kernel with key splits does not, so a step with a long portion sends all its rows to the former (behind
-        # a window no row walks far), and steps of short portions and decoded tokens go to the vector-unit kernel.
+        # The kernel that shares K and V tiles among four waves also takes kept first keys, the means of pooled
+        # blocks, and one more weight in a row's sum (of score 0: ``sinks`` all zero, which ``terms["zero_sink"]`` says
+        # without a look at the device; or of the head's own score); the per-wave kernel with key splits does not,
+        # so a step with a long portion sends all its rows to the former (behind a window no row walks far), and
+        # steps of short portions and decoded tokens go to the vector-unit kernel.
         zero_sink = bool(terms and terms.get("zero_sink")) and sinks is not None
-        windowed = (softcap == 0.0 and slopes is None and scale > 0 and (sinks is None or zero_sink)
-                    and (keep_first > 0 or zero_sink) and not pool)
+        windowed = (softcap == 0.0 and slopes is None and scale > 0
+                    and (keep_first > 0 or sinks is not None or pool > 0))
         if self.dtype == torch.bfloat16 and self.attention_mfma and (plain or windowed):
             gpl = max(0, (min(G, 16) - 1).bit_length())
             decode = getattr(ctx, "max_q_len", 1) == 1
@@ -360,7 +361,7 @@ class Attention:
                 if n32 >= th["four_waves_of_32_rows"] and D > 64:
                     wg_rt = 32
                 elif n32 >= th["eight_waves"]:
-                    wg_rt = 64 if not keep_first else 32      # (no kept keys with the keys in two halves)
+                    wg_rt = 64 if not (keep_first or pool) else 32      # (no kept keys or means with the keys in two halves)
             elif D <= 64 and (n_long // (4 * max(1, 32 >> gpl))) * Hkv * ((G + 15) // 16) >= th["two_tiles_of_16_rows"]:
                 wg_rt = 2
             wg_tokens = 4 * max(1, (32 if wg_rt >= 32 else 16 * wg_rt) >> gpl)
@@ -372,7 +373,7 @@ class Attention:
             # the row tiles (tests) forces the choice.
             enough = ((n_long // wg_tokens) * Hkv * ((G + 15) // 16) >= th["workgroup_kernel"]
                       or self.attention_row_tiles is not None)
-            if keep_first and wg_rt == 64:
+            if (keep_first or pool) and wg_rt == 64:
                 wg_rt = 32
             if (self.attention_workgroup and not decode and D <= 128 and self.attention_splits is None
                     and getattr(ctx, "max_q_len", 1) >= 16 and enough):
@@ -383,8 +384,10 @@ class Attention:
                     _ptr(q), _ptr(slot.k), _ptr(slot.v), _ptr(slot.block_table),
                     c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
                     c_int(n_blocks), _ptr(out), c_int(N), c_int(Hq), c_int(Hkv), c_int(slot.block_size),
-                    c_float(scale), c_int(w), c_int(rt), c_int(gpl), c_int(keep_first), c_int(1 if zero_sink else 0),
-                    self._stream()), "paged_attention (prefill)")
+                    c_float(scale), c_int(w), c_int(rt), c_int(gpl), c_int(keep_first),
+                    c_int(0 if sinks is None else (1 if zero_sink else 2)), _ptr(sinks),
+                    _ptr(means.k if pool else None), _ptr(means.v if pool else None), _ptr(means.block_table if pool else None),
+                    c_int(means.block_table.shape[1] if pool else 0), c_int(pool), self._stream()), "paged_attention (prefill)")
                 if mixed:
                     # after the long ones, on the same stream: side by side on a second stream
                     # was measured and is slower (35.4 ms against 32.3 ms per mixed step at 8B sizes)

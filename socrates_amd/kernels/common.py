@@ -84,7 +84,7 @@ _COMPOSITE_SIGNATURES = {
     "soc_window_prepare": [P, I, I, I, I, P, P, P, P, P, I, P, P, P, P, I, F, P, I, P, I, I, I, I, I, I, I, I, P],
     "soc_pool_blocks": [P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
     "soc_turn_back": [P, P, P, P, I, I, I, I, I, P],
-    "soc_linear_attention": [P, I, I, I, I, F, I, P, P, P, F, I, I, I, P, L, I, P, P, P, I, I, I, P],
+    "soc_linear_attention": [P, I, I, I, I, F, I, P, P, P, F, I, I, I, P, L, I, P, P, P, I, P, I, I, I, P],
     "soc_scaled_sum": [P, I, F, P, I, F, P, P, I, I, I, P],
     "soc_glu_gelu": [P, P, I, I, I, I, P],
 }
@@ -92,7 +92,7 @@ _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P
 _ATTENTION_SIGNATURES = {
     "soc_paged_attention_tokens": [P, P, P, P, I, P, P, P, P, P, I, I, I, I, F, I, I, I, I, F, P, P, I, P, P, P, I, I, P],
     "soc_paged_attention_mfma": [P, P, P, P, I, P, P, P, I, P, P, P, P, I, I, I, I, F, I, I, I, I, I, I, P],
-    "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, I, I, P],
+    "soc_paged_attention_prefill": [P, P, P, P, I, P, P, P, I, P, I, I, I, I, F, I, I, I, I, I, P, P, P, P, I, I, P],
     "soc_paged_attention_decode_fused": [P, I, P, P, P, I, P, P, P, P, P, P, I, I, I, I, F, I, I, I, I, P, P, P, F, I, I, P],
     "soc_attention_head_dim": [],
 }

@@ -18,6 +18,8 @@ _NORMS = {None: 0, "head": 1, "whole": 2}
 
 
 class Composite:
+    linear_prepare_ahead = 16       # tokens of a step's longest portion from which linear attention prepares ahead
+
     def _composite(self):
         lib = getattr(self, "_composite_lib", None)
         if lib is None:
@@ -168,11 +170,17 @@ class Composite:
             self._want(decays, "decays", torch.float32, (H,))
         stride = self._state(state, offset, H * D * Dv, ctx)
         out = torch.empty((N, H * Dv), dtype=torch.float32, device=self.device)
+        # a step with a portion of some length: activations, the scale and the decays are taken once, ahead of the
+        # walk (each of a head's workgroups would take them again); single tokens and short portions where they
+        # are staged
+        prep = None
+        if (activate or z is not None) and ctx.max_q_len >= self.linear_prepare_ahead:
+            prep = torch.empty((N, 3 if z is not None else 2, H * D), dtype=torch.float32, device=self.device)
         _check(self._composite().soc_linear_attention(
             _ptr(x), c_int(ld), c_int(col_q), c_int(col_k), c_int(col_v), c_float(q_scale), c_int(1 if activate else 0),
             _ptr(decays), _ptr(z), _ptr(z_bias), c_float(tau), c_int(H), c_int(D), c_int(Dv), _ptr(state), stride, c_int(offset),
-            _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), _ptr(out), c_int(ctx.n_seqs), c_int(ctx.max_q_len), c_int(self.code),
-            self._stream()), "linear_attention")
+            _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), _ptr(prep), c_int(N), _ptr(out), c_int(ctx.n_seqs), c_int(ctx.max_q_len),
+            c_int(self.code), self._stream()), "linear_attention")
         return out
 
     # -- sums and activations ----------------------------------------------------------------------------------------
