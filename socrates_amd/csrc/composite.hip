@@ -44,8 +44,9 @@ norm_add_cast_vec8_kernel(float* __restrict__ residual, const Y* __restrict__ y,
     for (int c = 0; c < C; ++c) {
         const int at = (threadIdx.x + c * 256) * 8;
         if (at < d) {
+            VecLoad<Y, 8>::load(y + row + at, v[c]);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { v[c][e] = to_float(y[row + at + e]); ss = fmaf(v[c][e], v[c][e], ss); }
+            for (int e = 0; e < 8; ++e) ss = fmaf(v[c][e], v[c][e], ss);
         }
     }
     ss = block_sum(ss, scratch);
@@ -54,11 +55,24 @@ norm_add_cast_vec8_kernel(float* __restrict__ residual, const Y* __restrict__ y,
     for (int c = 0; c < C; ++c) {
         const int at = (threadIdx.x + c * 256) * 8;
         if (at < d) {
+            float r[8], g[8];
+            VecLoad<float, 8>::load(residual + row + at, r);
+            VecLoad<float, 8>::load(gain + at, g);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float r = residual[row + at + e] + v[c][e] * inv * gain[at + e];
-                residual[row + at + e] = r;
-                if (out) out[row + at + e] = from_float<T>(r);
+            for (int e = 0; e < 8; ++e) r[e] += v[c][e] * inv * g[e];
+            *reinterpret_cast<float4*>(residual + row + at) = make_float4(r[0], r[1], r[2], r[3]);
+            *reinterpret_cast<float4*>(residual + row + at + 4) = make_float4(r[4], r[5], r[6], r[7]);
+            if (out) {
+                if constexpr (sizeof(T) == 2) {
+                    uint4 pk;
+                    pk.x = pack_bf16x2(r[0], r[1]); pk.y = pack_bf16x2(r[2], r[3]);
+                    pk.z = pack_bf16x2(r[4], r[5]); pk.w = pack_bf16x2(r[6], r[7]);
+                    *reinterpret_cast<uint4*>(out + row + at) = pk;
+                } else {
+                    float* of = reinterpret_cast<float*>(out + row + at);
+                    *reinterpret_cast<float4*>(of) = make_float4(r[0], r[1], r[2], r[3]);
+                    *reinterpret_cast<float4*>(of + 4) = make_float4(r[4], r[5], r[6], r[7]);
+                }
             }
         }
     }
@@ -137,8 +151,8 @@ SOC_EXPORT int soc_depth_average(float* residual, float* kept, int count, const 
 // [D]; 2: over the whole of q (gain [Hq D]) and the whole of k (gain [Hkv D]). Then elements 2i and 2i + 1 of the
 // first 2 * half of every q and k head are turned by position * inv_freq[i], and (value_freq given) elements 2m and
 // 2m + 1 of every v head by position * value_freq[m]. q goes to q_out [N, Hq, P], k and v to the token's place in the
-// pools [pages, Hkv, BS, P] (P even), zeros behind D and Dv. One workgroup per token; q and k pass through LDS (dynamic,
-// (Hq + Hkv) D floats).
+// pools [pages, Hkv, BS, P] (P even), zeros behind D and Dv. grid (tokens, groups of per heads); a workgroup's q and k
+// heads pass through LDS (dynamic, per * D floats).
 template <typename T>
 __global__ void __launch_bounds__(256)
 window_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int col_v, const float* __restrict__ bias,
@@ -146,32 +160,40 @@ window_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int
                       int table_width, const int* __restrict__ token_rows, const int* __restrict__ positions,
                       const float* __restrict__ q_gain, const float* __restrict__ k_gain, int norm, float eps,
                       const float* __restrict__ inv_freq, int half, const float* __restrict__ value_freq, int Hq, int Hkv,
-                      int D, int Dv, int P, int BS) {
-    extern __shared__ float qk[];                          // q heads, then k heads
+                      int D, int Dv, int P, int BS, int per) {
+    extern __shared__ float qk[];                          // the workgroup's heads: [per][D]
     __shared__ float scratch[16];
     const int n = blockIdx.x, tid = threadIdx.x;
     const int pos = positions[n];
     const T* row = x + (size_t)n * ld;
     const int nq = Hq * D, nk = Hkv * D;
-    for (int e = tid; e < nq + nk; e += 256) {
-        const int c = e < nq ? col_q + e : col_k + (e - nq);
-        qk[e] = to_float(row[c]) + (bias ? bias[c] : 0.f);
-    }
-    __syncthreads();
+    // the workgroup's heads among the Hq of q and, behind them, the Hkv of k (a k head brings its v head along)
+    const int h_lo = blockIdx.y * per, h_hi = min(Hq + Hkv, h_lo + per);
+    if (h_lo >= h_hi) return;
+    auto column = [&](int h, int i) { return h < Hq ? col_q + h * D + i : col_k + (h - Hq) * D + i; };
+    float iq = 1.f, ik = 1.f;
     if (norm == 2) {
+        // the statistics of the whole of q and of k: every workgroup of the token takes them for itself
         float sq = 0.f, sk = 0.f;
-        for (int e = tid; e < nq; e += 256) sq = fmaf(qk[e], qk[e], sq);
-        for (int e = tid; e < nk; e += 256) sk = fmaf(qk[nq + e], qk[nq + e], sk);
+        for (int e = tid; e < nq; e += 256) { const float v = to_float(row[col_q + e]) + (bias ? bias[col_q + e] : 0.f); sq = fmaf(v, v, sq); }
+        for (int e = tid; e < nk; e += 256) { const float v = to_float(row[col_k + e]) + (bias ? bias[col_k + e] : 0.f); sk = fmaf(v, v, sk); }
         sq = block_sum(sq, scratch);
         sk = block_sum(sk, scratch);
-        const float iq = 1.f / sqrtf(sq / (float)nq + eps), ik = 1.f / sqrtf(sk / (float)nk + eps);
-        for (int e = tid; e < nq; e += 256) qk[e] = qk[e] * iq * q_gain[e];
-        for (int e = tid; e < nk; e += 256) qk[nq + e] = qk[nq + e] * ik * k_gain[e];
-        __syncthreads();
-    } else if (norm == 1) {
+        iq = 1.f / sqrtf(sq / (float)nq + eps);
+        ik = 1.f / sqrtf(sk / (float)nk + eps);
+    }
+    for (int e = tid; e < (h_hi - h_lo) * D; e += 256) {
+        const int h = h_lo + e / D, i = e % D;
+        const int c = column(h, i);
+        float v = to_float(row[c]) + (bias ? bias[c] : 0.f);
+        if (norm == 2) v = h < Hq ? v * iq * q_gain[h * D + i] : v * ik * k_gain[(h - Hq) * D + i];
+        qk[e] = v;
+    }
+    __syncthreads();
+    if (norm == 1) {
         const int wave = tid / SOC_WAVE, lane = tid % SOC_WAVE;
-        for (int h = wave; h < Hq + Hkv; h += 256 / SOC_WAVE) {
-            float* head = qk + (size_t)h * D;
+        for (int h = h_lo + wave; h < h_hi; h += 256 / SOC_WAVE) {
+            float* head = qk + (size_t)(h - h_lo) * D;
             const float* gain = h < Hq ? q_gain : k_gain;
             float ss = 0.f;
             for (int i = lane; i < D; i += SOC_WAVE) ss = fmaf(head[i], head[i], ss);
@@ -189,18 +211,18 @@ window_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int
     if (g < lanes) {
         float sn = 0.f, cs = 1.f;
         if (j < half) sincosf((float)pos * inv_freq[j], &sn, &cs);
-        for (int h = g; h < Hq + Hkv; h += lanes) {
-            const float* head = qk + (size_t)h * D;
+        for (int h = h_lo + g; h < h_hi; h += lanes) {
+            const float* head = qk + (size_t)(h - h_lo) * D;
             const float a = 2 * j < D ? head[2 * j] : 0.f, b = 2 * j + 1 < D ? head[2 * j + 1] : 0.f;
             const float y0 = j < half ? a * cs - b * sn : a, y1 = j < half ? b * cs + a * sn : b;
             T* dst = h < Hq ? q_out + ((size_t)n * Hq + h) * P : k_pool + (place + (size_t)(h - Hq) * BS) * P;
             dst[2 * j] = from_float<T>(y0);
             dst[2 * j + 1] = from_float<T>(y1);
         }
-        // v heads
+        // the v heads of the workgroup's k heads
         sn = 0.f; cs = 1.f;
         if (value_freq && 2 * j + 1 < Dv) sincosf((float)pos * value_freq[j], &sn, &cs);
-        for (int h = g; h < Hkv; h += lanes) {
+        for (int h = max(h_lo, Hq) - Hq + g; h < h_hi - Hq; h += lanes) {
             const int c = col_v + h * Dv + 2 * j;
             const float a = 2 * j < Dv ? to_float(row[c]) + (bias ? bias[c] : 0.f) : 0.f;
             const float b = 2 * j + 1 < Dv ? to_float(row[c + 1]) + (bias ? bias[c + 1] : 0.f) : 0.f;
@@ -222,12 +244,21 @@ SOC_EXPORT int soc_window_prepare(const void* x, int ld, int col_q, int col_k, i
     if (norm && (!q_gain || !k_gain)) return (int)hipErrorInvalidValue;
     if (half && !inv_freq) return (int)hipErrorInvalidValue;
     if (value_freq && Dv % 2) return (int)hipErrorInvalidValue;
-    const size_t lds = (size_t)(Hq + Hkv) * D * sizeof(float);
+    // A token's heads go to as many workgroups as give the step about two per compute unit (a decode step has few
+    // tokens: one workgroup per token left the GPU idle), at most one per head.
+    int groups = (512 + N - 1) / N;
+    const int fit = (int)(((size_t)(Hq + Hkv) * D * sizeof(float) + 32 * 1024 - 1) / (32 * 1024));   // (and their heads fit LDS)
+    if (groups < fit) groups = fit;
+    if (groups > Hq + Hkv) groups = Hq + Hkv;
+    if (groups > 65535) groups = 65535;
+    const int per = (Hq + Hkv + groups - 1) / groups;
+    groups = (Hq + Hkv + per - 1) / per;
+    const size_t lds = (size_t)per * D * sizeof(float);
     if (lds > 60 * 1024) return (int)hipErrorInvalidValue;
 #define SOC_WP(T)                                                                                                             \
-    hipLaunchKernelGGL(window_prepare_kernel<T>, dim3(N), dim3(256), lds, stream, (const T*)x, ld, col_q, col_k, col_v, bias,  \
-                       (T*)q_out, (T*)k_pool, (T*)v_pool, table, table_width, token_rows, positions, q_gain, k_gain, norm,     \
-                       eps, inv_freq, half, value_freq, Hq, Hkv, D, Dv, P, BS)
+    hipLaunchKernelGGL(window_prepare_kernel<T>, dim3(N, groups), dim3(256), lds, stream, (const T*)x, ld, col_q, col_k,       \
+                       col_v, bias, (T*)q_out, (T*)k_pool, (T*)v_pool, table, table_width, token_rows, positions, q_gain,      \
+                       k_gain, norm, eps, inv_freq, half, value_freq, Hq, Hkv, D, Dv, P, BS, per)
     if (dtype == 0) SOC_WP(float); else SOC_WP(bf16);
 #undef SOC_WP
     return soc_last_error();

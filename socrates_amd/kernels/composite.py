@@ -85,8 +85,6 @@ class Composite:
             raise KernelError(f"head sizes {D} and {Dv} in pools of {P}, rotation over {rotary_dim}")
         if norm not in _NORMS:
             raise KernelError(f"norm {norm!r}: head, whole or None")
-        if (Hq + Hkv) * D * 4 > 60 * 1024:
-            raise KernelError(f"{Hq + Hkv} heads of {D}: queries and keys of a token do not fit a workgroup's LDS")
         if bias is not None:
             self._want(bias, "bias", torch.float32, (ld,))
         if norm is not None:
