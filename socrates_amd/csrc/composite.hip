@@ -267,14 +267,16 @@ SOC_EXPORT int soc_window_prepare(const void* x, int ld, int col_q, int col_k, i
 // ---- the means of the blocks that a step completes --------------------------------------------------------------
 // A sequence of the step that brings positions start .. end - 1 completes the blocks b with b * per + per - 1 among
 // them: start / per <= b < end / per. Mean key and mean value of block b, over the per tokens' entries in the pools
-// [pages, Hkv, BS, P] (summed in position order in float32), go to entry b of the row's pages of means
+// [pages, Hkv, BS, P] (summed in float32: every fourth position in order, then the four sums), go to entry b of the row's pages of means
 // (same shape, a table of their own). grid (blocks a sequence may complete, sequences, kv heads).
 template <typename T>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(256)
 pool_blocks_kernel(const T* __restrict__ k_pool, const T* __restrict__ v_pool, const int* __restrict__ table, int table_width,
                    T* __restrict__ mk_pool, T* __restrict__ mv_pool, const int* __restrict__ mtable, int mtable_width,
                    const int* __restrict__ seq_qstart, const int* __restrict__ seq_rows, const int* __restrict__ seq_ctx,
                    int Hkv, int P, int BS, int per) {
+    // four waves take every fourth position of the block each; their sums meet in LDS, in the waves' order
+    __shared__ float part_k[3][256], part_v[3][256];
     const int seq = blockIdx.y, kvh = blockIdx.z;
     const int n = seq_qstart[seq + 1] - seq_qstart[seq];
     const int end = seq_ctx[seq], start = end - n;
@@ -286,16 +288,26 @@ pool_blocks_kernel(const T* __restrict__ k_pool, const T* __restrict__ v_pool, c
     const int mpage = mtable[(size_t)row * mtable_width + b / BS];
     const size_t dst = (((size_t)mpage * Hkv + kvh) * BS + (size_t)(b % BS)) * P;
     const float inv = 1.f / (float)per;
-    for (int e = threadIdx.x; e < P; e += 64) {
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    for (int e0 = 0; e0 < P; e0 += 64) {                   // (P <= 256: the pools' head size)
+        const int e = e0 + lane;
         float sk = 0.f, sv = 0.f;
-        for (int t = 0; t < per; ++t) {
-            const int pos = b * per + t;
-            const size_t src = (((size_t)pages[pos / BS] * Hkv + kvh) * BS + (size_t)(pos % BS)) * P + e;
-            sk += to_float(k_pool[src]);
-            sv += to_float(v_pool[src]);
+        if (e < P) {
+            for (int t = wave; t < per; t += 4) {
+                const int pos = b * per + t;
+                const size_t src = (((size_t)pages[pos / BS] * Hkv + kvh) * BS + (size_t)(pos % BS)) * P + e;
+                sk += to_float(k_pool[src]);
+                sv += to_float(v_pool[src]);
+            }
         }
-        mk_pool[dst + e] = from_float<T>(sk * inv);
-        mv_pool[dst + e] = from_float<T>(sv * inv);
+        if (wave > 0) { part_k[wave - 1][e0 + lane] = sk; part_v[wave - 1][e0 + lane] = sv; }
+        __syncthreads();
+        if (wave == 0 && e < P) {
+#pragma unroll
+            for (int w = 0; w < 3; ++w) { sk += part_k[w][e0 + lane]; sv += part_v[w][e0 + lane]; }
+            mk_pool[dst + e] = from_float<T>(sk * inv);
+            mv_pool[dst + e] = from_float<T>(sv * inv);
+        }
     }
 }
 
@@ -304,10 +316,10 @@ SOC_EXPORT int soc_pool_blocks(const void* k_pool, const void* v_pool, const int
                                const int* seq_ctx, int n_seqs, int max_q_len, int Hkv, int P, int BS, int per, int dtype,
                                hipStream_t stream) {
     if (n_seqs <= 0) return 0;
-    if (per < 1 || BS < 1 || Hkv < 1 || P < 1 || n_seqs > 65535 || Hkv > 65535 || max_q_len < 1) return (int)hipErrorInvalidValue;
+    if (per < 1 || BS < 1 || Hkv < 1 || P < 1 || P > 256 || n_seqs > 65535 || Hkv > 65535 || max_q_len < 1) return (int)hipErrorInvalidValue;
     const dim3 grid(max_q_len / per + 1, n_seqs, Hkv);
 #define SOC_PB(T)                                                                                                              \
-    hipLaunchKernelGGL(pool_blocks_kernel<T>, grid, dim3(64), 0, stream, (const T*)k_pool, (const T*)v_pool, table, table_width, \
+    hipLaunchKernelGGL(pool_blocks_kernel<T>, grid, dim3(256), 0, stream, (const T*)k_pool, (const T*)v_pool, table, table_width, \
                        (T*)mk_pool, (T*)mv_pool, mtable, mtable_width, seq_qstart, seq_rows, seq_ctx, Hkv, P, BS, per)
     if (dtype == 0) SOC_PB(float); else SOC_PB(bf16);
 #undef SOC_PB
