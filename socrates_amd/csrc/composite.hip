@@ -12,11 +12,13 @@ __device__ __forceinline__ float cmp_sigmoid(float x) { return 1.f / (1.f + expf
 __device__ __forceinline__ float cmp_silu(float x) { return x * cmp_sigmoid(x); }
 
 // ---- residual += norm(y) * gain, and the sum in the compute dtype ---------------------------------------
-// One workgroup per row. y: the compute dtype or float32.
+// One workgroup per row. y: the compute dtype or float32. With kept ([total, n] float32, n = rows * d): the sum is the
+// layer's result, filed as kept[count], and what goes on (into residual and out) is sum over j <= count of w[j] kept[j],
+// in that order (the weighted sum over depth, below, in the same kernel).
 template <typename T, typename Y>
 __global__ void __launch_bounds__(256)
 norm_add_cast_kernel(float* __restrict__ residual, const Y* __restrict__ y, const float* __restrict__ gain, float eps,
-                     T* __restrict__ out, int d) {
+                     T* __restrict__ out, int d, float* __restrict__ kept, int count, const float* __restrict__ w, size_t n) {
     __shared__ float scratch[16];
     const size_t row = (size_t)blockIdx.x * d;
     float ss = 0.f;
@@ -24,7 +26,13 @@ norm_add_cast_kernel(float* __restrict__ residual, const Y* __restrict__ y, cons
     ss = block_sum(ss, scratch);
     const float inv = 1.f / sqrtf(ss / (float)d + eps);
     for (int c = threadIdx.x; c < d; c += 256) {
-        const float r = residual[row + c] + to_float(y[row + c]) * inv * gain[c];
+        float r = residual[row + c] + to_float(y[row + c]) * inv * gain[c];
+        if (kept) {                                        // the layer's result is filed, the weighted sum over depth goes on
+            kept[(size_t)count * n + row + c] = r;
+            float acc = 0.f;
+            for (int j = 0; j < count; ++j) acc = fmaf(w[j], kept[(size_t)j * n + row + c], acc);
+            r = fmaf(w[count], r, acc);
+        }
         residual[row + c] = r;
         if (out) out[row + c] = from_float<T>(r);
     }
@@ -35,7 +43,7 @@ norm_add_cast_kernel(float* __restrict__ residual, const Y* __restrict__ y, cons
 template <typename T, typename Y, int C>
 __global__ void __launch_bounds__(256)
 norm_add_cast_vec8_kernel(float* __restrict__ residual, const Y* __restrict__ y, const float* __restrict__ gain, float eps,
-                          T* __restrict__ out, int d) {
+                          T* __restrict__ out, int d, float* __restrict__ kept, int count, const float* __restrict__ w, size_t n) {
     __shared__ float scratch[16];
     const size_t row = (size_t)blockIdx.x * d;
     float v[C][8];
@@ -60,6 +68,24 @@ norm_add_cast_vec8_kernel(float* __restrict__ residual, const Y* __restrict__ y,
             VecLoad<float, 8>::load(gain + at, g);
 #pragma unroll
             for (int e = 0; e < 8; ++e) r[e] += v[c][e] * inv * g[e];
+            if (kept) {
+                float* own = kept + (size_t)count * n + row + at;
+                *reinterpret_cast<float4*>(own) = make_float4(r[0], r[1], r[2], r[3]);
+                *reinterpret_cast<float4*>(own + 4) = make_float4(r[4], r[5], r[6], r[7]);
+                float acc[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+                for (int j = 0; j < count; ++j) {
+                    float t[8];
+                    VecLoad<float, 8>::load(kept + (size_t)j * n + row + at, t);
+                    const float wj = w[j];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[e] = fmaf(wj, t[e], acc[e]);
+                }
+                const float wc = w[count];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) r[e] = fmaf(wc, r[e], acc[e]);
+            }
             *reinterpret_cast<float4*>(residual + row + at) = make_float4(r[0], r[1], r[2], r[3]);
             *reinterpret_cast<float4*>(residual + row + at + 4) = make_float4(r[4], r[5], r[6], r[7]);
             if (out) {
@@ -79,15 +105,16 @@ norm_add_cast_vec8_kernel(float* __restrict__ residual, const Y* __restrict__ y,
 }
 
 SOC_EXPORT int soc_norm_add_cast(float* residual, const void* y, int y_f32, const float* gain, float eps, void* out, int N,
-                                 int d, int dtype, hipStream_t stream) {
+                                 int d, float* kept, int count, const float* w, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (d < 1) return (int)hipErrorInvalidValue;
+    if (d < 1 || (kept && (count < 1 || !w))) return (int)hipErrorInvalidValue;
+    const size_t n = (size_t)N * d;
 #define SOC_NAC(T, Y)                                                                                                                \
     do {                                                                                                                             \
-        if (d % 8 == 0 && d <= 2048) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 1>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d);      \
-        else if (d % 8 == 0 && d <= 4096) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 2>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d); \
-        else if (d % 8 == 0 && d <= 8192) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 4>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d); \
-        else hipLaunchKernelGGL((norm_add_cast_kernel<T, Y>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d);                                     \
+        if (d % 8 == 0 && d <= 2048) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 1>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d, kept, count, w, n);      \
+        else if (d % 8 == 0 && d <= 4096) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 2>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d, kept, count, w, n); \
+        else if (d % 8 == 0 && d <= 8192) hipLaunchKernelGGL((norm_add_cast_vec8_kernel<T, Y, 4>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d, kept, count, w, n); \
+        else hipLaunchKernelGGL((norm_add_cast_kernel<T, Y>), dim3(N), dim3(256), 0, stream, residual, (const Y*)y, gain, eps, (T*)out, d, kept, count, w, n);                                     \
     } while (0)
     if (dtype == 0) SOC_NAC(float, float);
     else if (y_f32) SOC_NAC(bf16, float);

@@ -78,7 +78,7 @@ _HYBRID_SIGNATURES = {
     "soc_add_cast": [P, P, P, I, L, P, I, P],
 }
 _COMPOSITE_SIGNATURES = {
-    "soc_norm_add_cast": [P, P, I, P, F, P, I, I, I, P],
+    "soc_norm_add_cast": [P, P, I, P, F, P, I, I, P, I, P, I, P],
     "soc_depth_begin": [P, P, P, L, I, P],
     "soc_depth_average": [P, P, I, P, P, L, I, P],
     "soc_window_prepare": [P, I, I, I, I, P, P, P, P, P, I, P, P, P, P, I, F, P, I, P, I, I, I, I, I, I, I, I, P],

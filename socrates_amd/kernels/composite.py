@@ -38,30 +38,39 @@ class Composite:
                                                  c_int(self.code), self._stream()), "depth_begin")
         return (kept, out) if cast else kept
 
-    def norm_add_cast(self, residual, y, gain, eps, cast=True):
+    def norm_add_cast(self, residual, y, gain, eps, cast=True, depth=None):
         """residual (float32 [N, d], in place) += y / rms(y) * gain, y in the compute dtype or float32; with
-        ``cast`` returns the sum in the compute dtype."""
+        ``cast`` returns the sum in the compute dtype. ``depth`` = (kept, count, weights): that sum is a layer's
+        result; it is filed as kept[count] and what goes on, in residual and in what is returned, is the sum over
+        j <= count of weights[j] kept[j] (``depth_average`` in the same kernel)."""
         N, d = residual.shape
         self._want(residual, "residual", torch.float32)
         if y.dtype not in (self.dtype, torch.float32):
             raise KernelError(f"a branch's result in {y.dtype}")
         self._want(y, "branch result", y.dtype, (N, d))
         self._want(gain, "norm gain", torch.float32, (d,))
+        kept, count, weights = depth if depth is not None else (None, 0, None)
+        if depth is not None:
+            self._check_depth(kept, count, weights, N, d)
         out = torch.empty((N, d), dtype=self.dtype, device=self.device) if cast else None
         _check(self._composite().soc_norm_add_cast(_ptr(residual), _ptr(y), c_int(1 if y.dtype == torch.float32 else 0), _ptr(gain),
-                                                   c_float(eps), _ptr(out), c_int(N), c_int(d), c_int(self.code), self._stream()),
+                                                   c_float(eps), _ptr(out), c_int(N), c_int(d), _ptr(kept), c_int(count), _ptr(weights),
+                                                   c_int(self.code), self._stream()),
                "norm_add_cast")
         return out
+
+    def _check_depth(self, kept, count, weights, N, d):
+        self._want(kept, "results by depth", torch.float32)
+        if kept.dim() != 3 or tuple(kept.shape[1:]) != (N, d) or not 0 < count < kept.shape[0]:
+            raise KernelError(f"results by depth {tuple(kept.shape)} have no place {count} for rows of {(N, d)}")
+        self._want(weights, "depth weights", torch.float32, (count + 1,))
 
     def depth_average(self, residual, kept, count, weights, cast=True):
         """kept[count] <- residual; residual <- sum over j <= count of weights[j] kept[j]; with ``cast`` returns
         the sum in the compute dtype."""
         N, d = residual.shape
         self._want(residual, "residual", torch.float32)
-        self._want(kept, "results by depth", torch.float32)
-        if kept.dim() != 3 or tuple(kept.shape[1:]) != (N, d) or not 0 < count < kept.shape[0]:
-            raise KernelError(f"results by depth {tuple(kept.shape)} have no place {count} for rows of {(N, d)}")
-        self._want(weights, "depth weights", torch.float32, (count + 1,))
+        self._check_depth(kept, count, weights, N, d)
         out = torch.empty((N, d), dtype=self.dtype, device=self.device) if cast else None
         _check(self._composite().soc_depth_average(_ptr(residual), _ptr(kept), c_int(count), _ptr(weights), _ptr(out),
                                                    c_longlong(N * d), c_int(self.code), self._stream()), "depth_average")

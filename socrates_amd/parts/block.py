@@ -233,8 +233,9 @@ class DepthAverageBlock:
     itself; that x is the layer's result X_(i+1), and what goes on is sum_j w[j] X_j over the embedding
     output and all layers' results so far. The results are kept in float32 for the length of the step
     (``ctx.carry``: one tensor [layers + 1, N, d] that the first block of a step makes). One kernel norms
-    a branch's result, adds it to the stream and casts the sum for the part that reads it next; one more
-    files the layer's result, takes the weighted sum and casts it for the next layer's mixer."""
+    a branch's result, adds it to the stream and casts the sum for the part that reads it next; behind the
+    layer's last branch the same kernel files the layer's result, takes the weighted sum and casts it for
+    the next layer's mixer."""
     chains = True
     _CARRY = "results by depth"
 
@@ -276,11 +277,16 @@ class DepthAverageBlock:
                 ctx.carry[self._CARRY] = ops.depth_begin(residual, depth.n_layers + 1)
         kept = ctx.carry[self._CARRY]
         gain, eps = self.post1.fusable()
-        x = ops.norm_add_cast(residual, self.mixer.forward(x, ctx, slot, write), gain, eps, cast=self.ffn is not None)
-        if self.ffn is not None:
+        # the layer's last branch: its norm, the sum, the filing of the layer's result and the weighted sum over depth
+        # are one kernel, which also casts what goes on if the next block reads it as this one does
+        last = dict(cast=isinstance(nxt, DepthAverageBlock), depth=(kept, depth.index + 1, self.depth.weights))
+        y = self.mixer.forward(x, ctx, slot, write)
+        if self.ffn is None:
+            rows = ops.norm_add_cast(residual, y, gain, eps, **last)
+        else:
+            x = ops.norm_add_cast(residual, y, gain, eps, cast=True)
             gain, eps = self.post2.fusable()
-            ops.norm_add_cast(residual, self.ffn.forward(x, ctx), gain, eps, cast=False)
-        rows = ops.depth_average(residual, kept, depth.index + 1, self.depth.weights, cast=isinstance(nxt, DepthAverageBlock))
+            rows = ops.norm_add_cast(residual, self.ffn.forward(x, ctx), gain, eps, **last)
         return None if rows is None else Normed(rows)
 
 

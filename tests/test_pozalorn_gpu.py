@@ -251,6 +251,22 @@ def test_small_kernels(kernel_sets, dtype):
         _close(ops.depth_average(a, k1, count, w), ref.depth_average(b, k2, count, w), dtype, "weighted sum over depth")
         torch.testing.assert_close(a.cpu(), b.cpu(), atol=1e-5, rtol=1e-5)
         torch.testing.assert_close(k1[:count + 1].cpu(), k2[:count + 1].cpu(), atol=0, rtol=0)       # what has been filed so far
+    # a branch's norm and sum with the weighted sum over depth behind it, in one kernel; rows of 77 and of 2,560 elements
+    for d in (77, 2560):
+        r = torch.randn(9, d, generator=g).to(DEV)
+        gain_d = (1 + 0.3 * torch.randn(d, generator=g)).to(DEV)
+        k1, k2 = ops.depth_begin(r.clone(), 5), ref.depth_begin(r.clone(), 5)
+        for count, w in ((1, [0.3, -0.7]), (2, [0.1, 0.2, 0.5]), (3, [1.0, 0.0, -0.5, 0.25]), (4, [0.2, 0.2, 0.2, 0.2, 0.2])):
+            w = torch.tensor(w, device=DEV)
+            for wide in (False, True):
+                y = torch.randn(9, d, generator=g).to(torch.float32 if wide else dt).to(DEV)
+                a = torch.randn(9, d, generator=g).to(DEV)
+                b = a.clone()
+                got = ops.norm_add_cast(a, y, gain_d, 1e-5, cast=True, depth=(k1, count, w))
+                want = ref.norm_add_cast(b, y, gain_d, 1e-5, cast=True, depth=(k2, count, w))
+                _close(got, want, dtype, "norm, sum and the sum over depth")
+                torch.testing.assert_close(a.cpu(), b.cpu(), atol=2e-5, rtol=1e-5)
+                torch.testing.assert_close(k1[:count + 1].cpu(), k2[:count + 1].cpu(), atol=2e-5, rtol=1e-5)
     # the group norm with a sigmoid gate behind it
     y = torch.randn(33, 96, generator=g).to(DEV)
     zz = torch.randn(33, 96 + 5, generator=g).to(dt).to(DEV)
@@ -327,6 +343,35 @@ def test_a_wider_model_with_long_prompts(tmp_path, kernel_sets, dtype):
             compare(got[f"r{i}"], want[i], TOL[dtype], f"{name} {dtype} request {i}")
 
 
+@pytest.mark.parametrize("row_tiles", [1, 2, 32])
+def test_long_portions_through_the_prompt_kernel_on_the_matrix_cores(tmp_path, kernel_sets, row_tiles):
+    """bfloat16 steps whose long portions are sent to the prompt kernel on the matrix cores (by an override: models this
+    small have too few rows for it otherwise), with the cache manager's own pages, tables and pages of means: a
+    learned sink in one layer, pooled blocks in the other, whole prompts, portions behind cached tokens and single
+    tokens beside them, against the plain model."""
+    ops = kernel_sets["bfloat16"]
+    made = model(128, 300, [parallel(window(8, 2, 64, 64, 96, rot(64, 50000.0, (4.0, 1.0, 4.0, 2048)), scale=0.125),
+                                     lightning(2, 32, 32, (0.9, 0.99)), 0.8, 1.1),
+                            attention(4, 2, 64, 32, size=72, pool=16, rotation=rot(32, 250000.0, (8.0, 1.0, 4.0, 1024)), scale=0.125),
+                            gla(2, 32, 48, 16.0, rank=8)],
+                 [dense(256), dense(192), None])
+    folder = write_model(tmp_path / "m", made, seed=61)
+    prompts = random_prompts([400, 150, 333], made[0]["vocab"], seed=62)
+    want = oracle(folder, prompts)
+    ops.attention_row_tiles = row_tiles
+    try:
+        for name, steps in (("whole", CUTS["whole"](prompts)), ("mixed", trace_mixed(prompts, seed=63)),
+                            ("portions", trace_portions(prompts, seed=64, sizes=(17, 64, 65, 128, 200)))):
+            runner = make_runner(folder, ops, max_rows=4, max_len=448, block_size=16)
+            got = replay(runner, steps)
+            if name != "mixed":
+                assert ops.last_attention_kernel == ("workgroup", row_tiles)
+            for i in range(len(prompts)):
+                compare(got[f"r{i}"], want[i], TOL["bfloat16"], f"{name}, row tiles {row_tiles}, request {i}")
+    finally:
+        ops.attention_row_tiles = None
+
+
 @pytest.mark.parametrize("dtype", list(DTYPES))
 def test_edges_and_long_decoding(tmp_path, kernel_sets, dtype):
     """A window of 6 before which blocks of 4 come into sight, beside a window of 5 with sinks (in float32 under a
@@ -382,6 +427,36 @@ def test_greedy_generation_through_the_engine(folders, name):
                     block_size=BLOCK[name], chunk=16)
     assert engine.generate(prompts, max_new_tokens=8) == want
     engine.cache.check()
+
+
+def test_command_line(tmp_path, folders):
+    """``python -m socrates_amd.generate`` on a model folder, and with ``--random-weights`` on a configuration alone
+    (it writes a seeded random model into --model; the rank of the decays' inner projections, which only a tensor's
+    shape says, is made up): float32 greedy tokens are the plain model's."""
+    cfg, w = read_folder(folders["A"])
+    prompts = random_prompts([5, 17], cfg["vocab"], seed=2)
+    want = [plain.greedy(cfg, w, p, 5) for p in prompts]
+    cmd = [sys.executable, "-m", "socrates_amd.generate", "--model", str(folders["A"]), "--dtype", "float32",
+           "--max-new-tokens", "5", "--max-len", "64", "--max-batch", "2", "--block-size", "4"]
+    for p in prompts:
+        cmd += ["--prompt-ids", ",".join(map(str, p))]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300, cwd=str(ROOT))
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = proc.stdout.strip().split("\n")
+    shown = [l for i, l in enumerate(lines) if i > 0 and lines[i - 1].startswith("> ")]
+    assert shown == [" ".join(map(str, x)) for x in want]
+    (tmp_path / "config.json").write_text(json.dumps(MODELS["B"][0]))
+    made = tmp_path / "made"
+    cmd = [sys.executable, "-m", "socrates_amd.generate", "--model", str(made), "--random-weights", str(tmp_path / "config.json"),
+           "--seed", "4", "--dtype", "float32", "--max-new-tokens", "4", "--max-len", "64", "--max-batch", "2",
+           "--prompt-ids", "7,100,12,5,9"]
+    proc = subprocess.run(cmd, capture_output=True, text=True, timeout=300, cwd=str(ROOT))
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    cfg, w = read_folder(made)
+    assert cfg == MODELS["B"][0] and w["l2.mix.a1"].shape[1] == cfg["width"]
+    lines = proc.stdout.strip().split("\n")
+    shown = [l for i, l in enumerate(lines) if i > 0 and lines[i - 1].startswith("> ")]
+    assert shown == [" ".join(map(str, plain.greedy(cfg, w, [7, 100, 12, 5, 9], 4)))]
 
 
 def test_trace_runner_on_a_model_folder(tmp_path, folders):

@@ -431,8 +431,10 @@ class TorchKernels:
         kept[0] = residual
         return (kept, residual.to(self.dtype)) if cast else kept
 
-    def norm_add_cast(self, residual, y, gain, eps, cast=True):
+    def norm_add_cast(self, residual, y, gain, eps, cast=True, depth=None):
         residual += self._norm(y, gain, eps).to(residual.dtype)
+        if depth is not None:
+            return self.depth_average(residual, *depth, cast=cast)
         return residual.to(self.dtype) if cast else None
 
     def depth_average(self, residual, kept, count, weights, cast=True):
