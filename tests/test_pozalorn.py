@@ -387,3 +387,27 @@ def test_greedy_generation_through_the_engine(folders):
     engine = Engine(runner, device="cpu", dtype=torch.float32, compile=False, max_batch=3, max_len=64, max_new_tokens=6,
                     block_size=4, chunk=8)
     assert engine.generate(prompts, max_new_tokens=6) == want
+
+
+def test_tokens_do_not_depend_on_the_pool(folders):
+    """Pools so small that requests wait and have their portions shortened, and two requests that fit at admission and
+    outgrow the pool while decoding behind a window longer than they are: the younger is preempted and computed again
+    (its states cleared, its means taken anew). float64 greedy tokens are those of a roomy pool and of the plain model."""
+    from socrates_amd.engine import Engine
+    cfg, w = read_folder(folders["B"])
+    prompts = random_prompts([5, 17, 33, 9, 24, 40, 1, 12], cfg["vocab"], seed=27)
+    want = [plain.greedy(cfg, w, p, 8) for p in prompts]
+
+    def engine_with(num_blocks, chunk):
+        runner = make_runner(folders["B"], ops64(), max_rows=4, max_len=64, block_size=4, num_blocks=num_blocks)
+        return Engine(runner, device="cpu", dtype=torch.float64, compile=False, max_batch=4, max_len=64, max_new_tokens=8,
+                      block_size=4, chunk=chunk)
+    for num_blocks, chunk in ((64, 2048), (14, 7), (12, 5)):
+        engine = engine_with(num_blocks, chunk)
+        assert engine.generate(prompts, max_new_tokens=8) == want, (num_blocks, chunk)
+        engine.cache.check()
+        assert not engine.cache.open_rows and all(g.allocator.n_free == g.allocator.num_blocks for g in engine.cache.groups)
+    engine = engine_with(7, 64)
+    assert engine.generate([prompts[7], prompts[3]], max_new_tokens=8) == [want[7], want[3]]
+    assert engine.scheduler.n_preemptions > 0
+    engine.cache.check()
