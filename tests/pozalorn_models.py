@@ -69,16 +69,16 @@ STRETCH = (4.0, 1.0, 4.0, 64)           # wavelengths of 16 to 64 positions slid
 ONE_GLA = model(40, 61, [gla(3, 12, 20, 8.0, rank=5)], [dense(56)])
 ONE_POOLED = model(48, 53, [attention(4, 2, 24, 12, size=7, pool=3, rotation=rot(8, 1000.0, STRETCH), scale=0.3)], [dense(40)], eps=1e-6)
 ONE_PARALLEL = model(56, 67, [parallel(window(6, 3, 8, 20, 9, rot(8, 500.0)), lightning(2, 12, 16, (0.9, 0.99)), 0.6, 1.3)], [None])
-MIX_A = model(64, 97, [gla(2, 16, 32, 16.0, rank=4),
-                       attention(3, 1, 32, 16, size=9, pool=4, rotation=rot(16, 250000.0, (8.0, 1.0, 4.0, 32)), scale=0.2),
-                       parallel(window(4, 2, 16, 24, 5, rot(16, 10000.0, STRETCH), scale=0.4), lightning(3, 8, 8, (0.5, 0.97, 1.0)), 0.8, 1.1),
+MIX_A = model(64, 97, [gla(2, 16, 32, 12.0, rank=4),
+                       attention(3, 1, 32, 16, size=9, pool=4, rotation=rot(16, 300000.0, (6.0, 1.0, 4.0, 32)), scale=0.2),
+                       parallel(window(4, 2, 16, 24, 5, rot(16, 10000.0, STRETCH), scale=0.4), lightning(3, 8, 8, (0.5, 0.97, 1.0)), 0.7, 1.2),
                        attention(2, 2, 40, 24, size=12, pool=16, rotation=rot(20), scale=0.15),
                        gla(4, 8, 8, 1.0, rank=9)],
               [dense(80), None, dense(48), dense(100), None])
-MIX_B = model(96, 130, [parallel(window(8, 2, 16, 16, 200, rot(16, 250000.0)), lightning(1, 48, 80, (0.98,)), 1.0, 1.0),
+MIX_B = model(96, 130, [parallel(window(8, 2, 16, 16, 200, rot(16, 300000.0)), lightning(1, 48, 80, (0.98,)), 1.0, 1.0),
                         attention(6, 2, 48, 16, size=33, pool=5, rotation=rot(24, 100.0, (2.0, 1.0, 8.0, 128)), scale=0.1),
                         gla(1, 48, 80, 4.0, rank=16),
-                        parallel(window(3, 3, 32, 8, 17, rot(4, 50000.0, STRETCH), scale=0.25), lightning(5, 4, 12, (0.6, 0.8, 0.9, 0.95, 0.999)), 1.5, 0.4)],
+                        parallel(window(3, 3, 32, 8, 17, rot(4, 40000.0, STRETCH), scale=0.25), lightning(5, 4, 12, (0.6, 0.8, 0.9, 0.95, 0.999)), 1.5, 0.4)],
               [dense(200), dense(24), None, dense(64)], eps=3e-6)
 MODELS = {"gla": ONE_GLA, "pooled": ONE_POOLED, "parallel": ONE_PARALLEL, "A": MIX_A, "B": MIX_B}
 BLOCK = {"gla": 16, "pooled": 4, "parallel": 4, "A": 4, "B": 16}

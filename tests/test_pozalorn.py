@@ -83,7 +83,7 @@ def test_configuration_errors():
 
 
 # ---- each mechanism of the stand-in kernel set against the plain function ---------------------------------
-@pytest.mark.parametrize("dims,base,stretch", [(16, 250000.0, (8.0, 1.0, 4.0, 32)), (64, 50000.0, (4.0, 1.0, 4.0, 2048)), (8, 100.0, None),
+@pytest.mark.parametrize("dims,base,stretch", [(16, 300000.0, (6.0, 1.0, 4.0, 32)), (48, 40000.0, (3.0, 1.0, 8.0, 4096)), (8, 100.0, None),
                                                (24, 10000.0, (2.0, 2.0, 16.0, 64)), (2, 7.0, (3.0, 1.0, 2.0, 4))])
 def test_stretched_frequencies(dims, base, stretch):
     """Short wavelengths stay, long ones are divided, and those between slide from the one to the other."""

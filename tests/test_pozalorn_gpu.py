@@ -142,7 +142,7 @@ def _pooled_slot(dt, Hkv, P, bs, per, rows, pages, g):
 
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
-@pytest.mark.parametrize("window,per,bs", [(5, 4, 4), (7, 3, 4), (40, 16, 16), (3, 1, 4), (6, 7, 4), (9, 5, 16), (72, 16, 16)])
+@pytest.mark.parametrize("window,per,bs", [(5, 4, 4), (7, 3, 4), (40, 16, 16), (3, 1, 4), (6, 7, 4), (9, 5, 16), (88, 8, 16)])
 def test_pooled_blocks_in_the_attention_kernels(kernel_sets, dtype, window, per, bs):
     """The means of the blocks that a step completes, from the pages (blocks that span pages, pages that span
     blocks), then the paged-attention kernel with the visible means in front of the window, against the stand-in:
@@ -182,7 +182,7 @@ def test_pooled_blocks_in_the_attention_kernels(kernel_sets, dtype, window, per,
 
 @pytest.mark.parametrize("row_tiles", [None, 1, 2, 32])
 @pytest.mark.parametrize("window,per,P,G", [(40, 7, 32, 2), (100, 16, 64, 1), (64, 64, 128, 4), (7, 1, 48, 2), (500, 3, 64, 2), (33, 100, 32, 1),
-                                           (72, 16, 64, 2)])
+                                           (88, 8, 64, 2)])
 def test_prompt_attention_on_the_matrix_cores_sees_the_pooled_blocks(kernel_sets, window, per, P, G, row_tiles):
     """Long portions go to the kernel that shares its key tiles among four waves: the means of the blocks before the
     window in tiles of their own in front of the window's, with and without a learned sink per head, rows of several
@@ -324,10 +324,10 @@ def test_a_wider_model_with_long_prompts(tmp_path, kernel_sets, dtype):
     """Width 320, five layers, keys of 80 beside values of 48 and of 32 beside 112, states of 64 x 96 and 128 x 32,
     windows of 100, 37 and 300 with blocks of 16 and 10, prompts of up to 700 tokens: decoded at the end, mixed,
     and in portions of 2 to 200 tokens, through captured decode steps."""
-    made = model(320, 500, [parallel(window(10, 5, 80, 48, 100, rot(40, 50000.0, (4.0, 1.0, 4.0, 256)), scale=0.1),
-                                     lightning(5, 64, 96, (0.9, 0.97, 0.99, 0.995, 0.999)), 0.8, 1.1),
-                            gla(5, 64, 96, 16.0, rank=16),
-                            attention(4, 1, 32, 112, size=37, pool=10, rotation=rot(32, 250000.0, (8.0, 1.0, 4.0, 128)), scale=0.2),
+    made = model(320, 500, [parallel(window(10, 5, 80, 48, 100, rot(40, 40000.0, (3.0, 1.0, 4.0, 256)), scale=0.1),
+                                     lightning(5, 64, 96, (0.9, 0.97, 0.99, 0.995, 0.999)), 0.7, 1.2),
+                            gla(5, 64, 96, 12.0, rank=16),
+                            attention(4, 1, 32, 112, size=37, pool=10, rotation=rot(32, 300000.0, (6.0, 1.0, 4.0, 128)), scale=0.2),
                             attention(5, 5, 64, 48, size=300, pool=16, rotation=rot(64, 1e6), scale=0.12),
                             gla(2, 128, 32, 4.0, rank=7)],
                  [dense(520), dense(100), None, dense(640), dense(320)])
@@ -350,10 +350,10 @@ def test_long_portions_through_the_prompt_kernel_on_the_matrix_cores(tmp_path, k
     learned sink in one layer, pooled blocks in the other, whole prompts, portions behind cached tokens and single
     tokens beside them, against the plain model."""
     ops = kernel_sets["bfloat16"]
-    made = model(128, 300, [parallel(window(8, 2, 64, 64, 96, rot(64, 50000.0, (4.0, 1.0, 4.0, 2048)), scale=0.125),
-                                     lightning(2, 32, 32, (0.9, 0.99)), 0.8, 1.1),
-                            attention(4, 2, 64, 32, size=72, pool=16, rotation=rot(32, 250000.0, (8.0, 1.0, 4.0, 1024)), scale=0.125),
-                            gla(2, 32, 48, 16.0, rank=8)],
+    made = model(128, 300, [parallel(window(6, 3, 64, 32, 80, rot(48, 20000.0, (3.0, 1.0, 8.0, 512)), scale=0.15),
+                                     lightning(2, 32, 48, (0.9, 0.99)), 0.7, 1.2),
+                            attention(6, 2, 32, 64, size=56, pool=24, rotation=rot(32, 300000.0, (6.0, 1.0, 4.0, 256)), scale=0.2),
+                            gla(2, 32, 48, 8.0, rank=8)],
                  [dense(256), dense(192), None])
     folder = write_model(tmp_path / "m", made, seed=61)
     prompts = random_prompts([400, 150, 333], made[0]["vocab"], seed=62)
