@@ -64,7 +64,7 @@ __device__ __forceinline__ void merge_partial(float& m, float& l, float (&a)[EPL
 //   keep_first  with a window: the keys at positions below keep_first stay visible to every later token,
 //            at their true positions (a token then walks those keys, then its window)
 //   pool     > 0, with a window: before its window a token sees one mean key and value for every block of
-//            pool positions that lies wholly before the window (block b if b * pool + pool - 1 <= p - window);
+//            pool positions that ends before the window begins (block b if b * pool + pool - 1 <= p - window);
 //            entry b of the row's pages of means (mean_k, mean_v: pools of the cache's shape, with a table of
 //            their own) holds them. A token then walks those entries, then its window. Not with keep_first.
 struct ScoreTerms {
@@ -80,7 +80,7 @@ struct ScoreTerms {
 };
 
 // How many entries a token at position p walks before its window (which starts at lo): kept first keys, or the
-// means of the blocks that lie wholly before the window.
+// means of the blocks that end before the window begins.
 __device__ __forceinline__ int walk_prefix(const ScoreTerms& st, int p, int window, int lo) {
     if (st.pool > 0) return window > 0 ? max(0, (p - window + 1) / st.pool) : 0;
     return min(st.keep_first, lo);
@@ -1175,7 +1175,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     int kept = window > 0 ? min(keep_first, kmin) : 0, n_pre = (kept + PF_KEYS - 1) / PF_KEYS;
     if (n_pre * PF_KEYS > (kmin & ~(PF_KEYS - 1))) { kmin = 0; kept = 0; n_pre = 0; }
     // With pooled blocks (pool > 0, a window, no kept keys) the tiles in front of the window's hold the means of the
-    // blocks of pool positions that lie wholly before a row's window, from pages of their own: entry e of the row's
+    // blocks of pool positions that end before a row's window begins, from pages of their own: entry e of the row's
     // pages of means is walked as the key PF_MEAN + e (negative, so a tile of means is known by its first key), and
     // the row at position p sees the entries below (p - window + 1) / pool.
     auto blocks_before = [&](int pos) { const int d = pos - window + 1; return d > 0 ? d / pool : 0; };
@@ -1629,7 +1629,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 // row_tiles 64: the same with eight waves, four for each half of a block's keys. keep_first (with a window): the
 // keys below it stay visible to every row (not with row_tiles 64); sink 1: one more weight of score 0 and no value
 // in every row's sum; sink 2: of the score sinks[head] (not scaled). pool > 0 (with a window, not with kept keys or
-// row_tiles 64): a row also sees the means of the blocks of pool positions that lie wholly before its window, entries
+// row_tiles 64): a row also sees the means of the blocks of pool positions that end before its window begins, entries
 // of the pools mean_k, mean_v (pages of BS entries, table mean_table).
 SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, const void* v_pool,
                                            const int* block_table, int table_width, const int* token_rows,

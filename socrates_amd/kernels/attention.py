@@ -278,7 +278,7 @@ class Attention:
         slope * (key position - query position) added to the scaled scores) and ``keep_first``
         (int, with a window: the keys at positions below it stay visible to every later token) and ``pooled`` (the
         cache slot, whose pages of means hold one mean key and value per block of ``slot.pool`` positions: a token sees
-        the blocks that lie wholly before its window, in the same softmax). Such a layer,
+        the blocks that end before its window begins, in the same softmax). Such a layer,
         and one whose scale is not positive, goes to the kernel that computes scores on the
         vector units, in either dtype; the MFMA kernels take plain scores only."""
         N, Hq, D = q.shape

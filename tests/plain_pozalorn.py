@@ -57,7 +57,7 @@ def turn_pairs(x, positions, dims, freq, sign=1.0):
 
 
 def linear_attention(q, k, v, decay):
-    """S_t = diag(decay_t) S_(t-1) + k_t v_t^T (the decay on the rows that belong to key channels),
+    """S_t = diag(decay_t) S_(t-1) + k_t v_t^T (row i of a head's state is scaled by the decay of key channel i),
     o_t = S_t^T q_t. q, k [T, H, D], v [T, H, Dv], decay [T, H, D]."""
     T, H, D = q.shape
     S = torch.zeros(H, D, v.shape[-1], dtype=F)
@@ -138,7 +138,7 @@ def window_attention(h, W, m, eps):
 
 def pooled_attention(h, W, m, eps):
     """Softmax attention over a window and, before it, one mean key and value per block of tokens that
-    lies wholly before the window; q and k normed over the whole projection; values turned by their
+    ends before the window begins; q and k normed over the whole projection; values turned by their
     position and the result turned back by the query's."""
     T = h.shape[0]
     H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]

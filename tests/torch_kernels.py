@@ -149,7 +149,7 @@ class TorchKernels:
             k = slot.k[pages, :, offs].to(self.acc)          # [n, Hkv, D]
             v = slot.v[pages, :, offs].to(self.acc)
             if terms.get("pooled") is not None and window is not None:
-                # the means of the blocks that lie wholly before the window, in front of the window's keys
+                # the means of the blocks that end before the window begins, in front of the window's keys
                 means, per = terms["pooled"].pooled, terms["pooled"].pool
                 blocks = np.arange(max(0, (p - window + 1) // per))
                 mtable = means.block_table.cpu().numpy()
