@@ -11,6 +11,7 @@ from __future__ import annotations
 import json
 from pathlib import Path
 
+from .berelorn import BerelornConfig
 from .mitisun import MitisunConfig
 from .pozalorn import PozalornConfig
 from .qwen3 import ConfigError, Qwen3Config
@@ -102,3 +103,4 @@ register_architecture("Qwen3ForCausalLM", Qwen3Config)
 register_architecture("Mitisun", MitisunConfig)
 register_architecture("Tedulorn", TedulornConfig)
 register_architecture("Pozalorn", PozalornConfig)
+register_architecture("Berelorn", BerelornConfig)

@@ -84,9 +84,10 @@ class AttentionSpec:
 
 @dataclass(frozen=True)
 class SwiGLUSpec:
-    """y = Wd((Wu x) * silu(Wg x)), no bias."""
+    """y = Wd((Wu x) * silu(Wg x)), no bias. ``names``: the local names of Wg, Wu and Wd on disk."""
     hidden: int
     intermediate: int
+    names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
 
 
 @dataclass(frozen=True)
@@ -107,8 +108,19 @@ class PairRopeSpec:
     # by factor, one whose wavelength is shorter than original / high stays, and between the two, with
     # s = (original / wavelength - low) / (high - low), it becomes (1 - s) f / factor + s f. None: no stretch.
     stretch: Optional[Tuple[float, float, float, float]] = None
+    # (factor, original, fast, slow): the stretch as a linear ramp over the pair index. With
+    # index(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(index(fast)), 0) and
+    # hi = min(ceil(index(slow)), dims - 1), pair i has r = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) and the
+    # frequency r f / factor + (1 - r) f; cosines and sines are multiplied by 0.1 ln(factor) + 1 (``magnitude``).
+    ramp: Optional[Tuple[float, float, float, float]] = None
 
     def __post_init__(self):
+        if self.stretch is not None and self.ramp is not None:
+            raise ValueError("a rotation is stretched by wavelength or by a ramp over the pair index, not both")
+        if self.ramp is not None:
+            factor, original, fast, slow = self.ramp
+            if not (factor > 0 and original > 0 and fast > 0 and slow > 0 and self.base > 1):
+                raise ValueError(f"ramp (factor, original, fast, slow) = {self.ramp}: all positive, over a base above 1")
         if self.dims < 2 or self.dims % 2:
             raise ValueError(f"a rotation over pairs needs an even number of dimensions, not {self.dims}")
         if not self.base > 0:
@@ -134,7 +146,23 @@ class PairRopeSpec:
                     t = (original / wave - low) / (high - low)
                     f = (1.0 - t) * f / factor + t * f
             out.append(f)
+        if self.ramp is not None:
+            factor, original, fast, slow = self.ramp
+
+            def index(turns):
+                return self.dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
+            lo = max(math.floor(index(fast)), 0)
+            hi = min(math.ceil(index(slow)), self.dims - 1)
+            for i, f in enumerate(out):
+                r = min(1.0, max(0.0, (i - lo) / max(hi - lo, 0.001)))
+                out[i] = r * f / factor + (1.0 - r) * f
         return out
+
+    @property
+    def magnitude(self) -> float:
+        """What cosines and sines are multiplied by (1 without a ramp)."""
+        import math
+        return 1.0 if self.ramp is None else 0.1 * math.log(self.ramp[0]) + 1.0
 
 
 @dataclass(frozen=True)
@@ -337,18 +365,33 @@ class RoutedExpertsSpec:
     ``corrected`` False: by s). Experts form ``n_groups`` equal groups of neighbours; a group's score is
     its largest choice score, and only experts of the ``keep_groups`` best groups can be chosen. The
     weights are the chosen experts' s over their sum (+ ``renorm_eps``). ``shared``: one more such
-    feed-forward that every token uses, added unweighted (None: none)."""
+    feed-forward that every token uses, added unweighted (None: none).
+
+    ``scoring`` "sigmoid": s = sigmoid(W_router x) in place of the softmax. ``group_top`` = n: a group's score is the
+    sum of its n largest choice scores (1: its largest). ``scale``: the weights are multiplied by it. ``expert`` and
+    ``shared`` may also be a ``SwiGLUSpec`` (a plain silu gate, no clamp). ``shared_gate``: the shared expert's
+    result is multiplied by sigmoid(w_sg . x), one number per token (stored as ``shared.sg`` [1, hidden])."""
     hidden: int
     n_experts: int
     top: int
-    expert: ClampedGLUSpec
+    expert: object
     n_groups: int = 1
     keep_groups: int = 1
-    shared: Optional[ClampedGLUSpec] = None
+    shared: object = None
     corrected: bool = True
     renorm_eps: float = 1e-20
+    scoring: str = "softmax"
+    group_top: int = 1
+    scale: float = 1.0
+    shared_gate: bool = False
 
     def __post_init__(self):
+        if self.scoring not in ("softmax", "sigmoid"):
+            raise ValueError(f"scoring {self.scoring!r}: softmax or sigmoid")
+        if self.group_top < 1:
+            raise ValueError("a group's score sums at least its largest score")
+        if self.shared_gate and self.shared is None:
+            raise ValueError("a gate on the shared expert needs a shared expert")
         if not 1 <= self.top <= self.n_experts:
             raise ValueError(f"a token uses {self.top} of {self.n_experts} experts")
         if self.n_groups < 1 or self.n_experts % self.n_groups or not 1 <= self.keep_groups <= self.n_groups:
@@ -383,7 +426,13 @@ class WindowAttentionSpec:
     back by i (None: values as they are). A query at position i sees key j with
     0 <= i - j < ``window`` (None: all j <= i) and, with ``pool`` = P > 0, one mean key and mean value (of
     what the cache holds) for every block bP .. bP + P - 1 with bP + P - 1 <= i - window, in the same
-    softmax. ``sinks``: a stored number per head whose exponential joins the softmax's denominator."""
+    softmax. ``sinks``: a stored number per head whose exponential joins the softmax's denominator.
+
+    ``qk_norm`` "turned": q and k are divided by their root mean square per head after the rotation, with no gain.
+    ``tied_values``: there is no value projection; a token's values are its keys as projected, before norm and
+    rotation (v_dim equals head_dim). ``softcap`` = c: a scaled score s becomes c tanh(s / c). ``head_gate``: head
+    h's result is multiplied by sigmoid(W_g x)_h (stored as ``g`` [heads, hidden]) before the output projection.
+    ``keep_first``: with a window, the keys at positions below it stay visible to every later token."""
     hidden: int
     n_heads: int
     n_kv_heads: int
@@ -399,16 +448,26 @@ class WindowAttentionSpec:
     qkv_bias: bool = False
     o_bias: bool = False
     value_base: Optional[float] = None
+    tied_values: bool = False
+    softcap: Optional[float] = None
+    head_gate: bool = False
+    keep_first: int = 0
 
     def __post_init__(self):
         if self.n_heads < 1 or self.n_kv_heads < 1 or self.n_heads % self.n_kv_heads:
             raise ValueError(f"n_heads {self.n_heads} is not a multiple of n_kv_heads {self.n_kv_heads}")
         if not 1 <= self.head_dim <= 256 or not 1 <= self.v_dim <= 256:
             raise ValueError(f"head sizes {self.head_dim} and {self.v_dim}: the attention kernels take up to 256")
-        if self.qk_norm not in (None, "head", "whole"):
-            raise ValueError(f"qk_norm {self.qk_norm!r}: head, whole or None")
+        if self.qk_norm not in (None, "head", "whole", "turned"):
+            raise ValueError(f"qk_norm {self.qk_norm!r}: head, whole, turned or None")
         if self.window is not None and self.window < 1:
             raise ValueError("window must be at least 1")
+        if self.tied_values and (self.v_dim != self.head_dim or self.value_base is not None):
+            raise ValueError("values that are the keys have the keys' size and are not turned")
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError("softcap must be positive")
+        if self.keep_first < 0 or (self.keep_first and self.pool):
+            raise ValueError("keep_first is not negative, and not combined with pooled blocks")
         if self.pool < 0 or (self.pool and self.window is None):
             raise ValueError("pooled blocks lie before a window: pool needs a window and is not negative")
         if self.position is not None and self.position.dims > self.head_dim:
@@ -423,6 +482,90 @@ class WindowAttentionSpec:
         """Elements per cached key and per cached value: the larger of the two sizes, padded to the
         kernels' step."""
         return (max(self.head_dim, self.v_dim) + 15) // 16 * 16
+
+
+@dataclass(frozen=True)
+class DifferentialAttentionSpec:
+    """Grouped-query attention with two softmax maps per head over the same values, the second subtracted.
+
+    q holds, head by head, [map 1 | map 2] of ``head_dim`` each, k likewise per kv head; v [kv heads x ``v_dim``];
+    all three and the output projection with biases. ``position`` turns interleaved pairs of every map of q and k.
+    Query i sees key j <= i if i - j < ``window`` or j < ``keep_first`` (``window`` None: all). With a1, a2 the two
+    maps' results and lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + ``diff`` (four stored vectors of head_dim), a head's
+    result is (a1 - lambda a2) over its root mean square (eps inside the root, no gain) times (1 - diff).
+    ``own_kv`` False: the layer has no k and v projections and reads the cache slot another such layer writes.
+    ``cache_window`` / ``cache_keep_first``: what the cache slot has to hold, the widest of all layers that read it
+    (``cache_window`` 0: this layer's own window and kept keys; None: every position)."""
+    hidden: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    v_dim: int
+    scale: float
+    eps: float
+    diff: float
+    position: Optional[PairRopeSpec] = None
+    window: Optional[int] = None
+    keep_first: int = 0
+    own_kv: bool = True
+    cache_window: Optional[int] = 0
+    cache_keep_first: int = 0
+
+    @property
+    def cache_mask(self):
+        """(window, kept first keys) of what the cache slot holds."""
+        if self.cache_window == 0:
+            return self.window, (self.keep_first if self.window is not None else 0)
+        return self.cache_window, (self.cache_keep_first if self.cache_window is not None else 0)
+
+    def __post_init__(self):
+        if self.n_heads < 1 or self.n_kv_heads < 1 or self.n_heads % self.n_kv_heads:
+            raise ValueError(f"n_heads {self.n_heads} is not a multiple of n_kv_heads {self.n_kv_heads}")
+        if not 1 <= self.head_dim <= 256 or not 1 <= self.v_dim <= 256:
+            raise ValueError(f"head sizes {self.head_dim} and {self.v_dim}: the attention kernels take up to 256")
+        if self.window is not None and self.window < 1:
+            raise ValueError("window must be at least 1")
+        if self.keep_first < 0 or self.cache_keep_first < 0 or (self.cache_window is not None and self.cache_window < 0):
+            raise ValueError("keep_first and cache_window are not negative")
+        if self.position is not None and self.position.dims > self.head_dim:
+            raise ValueError(f"the rotation covers {self.position.dims} dimensions, a map has {self.head_dim}")
+        if not self.scale > 0:
+            raise ValueError("scale must be positive")
+        if self.window is None:
+            if self.cache_window:
+                raise ValueError("the cache must keep every position for a layer without a window")
+        elif self.cache_window and (self.cache_window < self.window or
+                                    (self.keep_first and self.cache_keep_first < self.keep_first)):
+            raise ValueError("the cache must keep at least the layer's own window and first keys")
+
+    @property
+    def cache_width(self) -> int:
+        """Elements per cached key and per cached value: the larger of the two sizes, padded to the
+        kernels' step."""
+        return (max(self.head_dim, self.v_dim) + 15) // 16 * 16
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """A matrix memory per head with exponential gates (mLSTM). q = Wq h * head_dim^-1/2, k = Wk h, v = Wv h; per
+    head a log input gate i = cap tanh((Wi h + bi) / cap) and a log forget gate f = logsigmoid(cap tanh((Wf h + bf) /
+    cap)); with a running maximum m (0 at the start): m' = max(f + m, i), S <- exp(f + m - m') S + exp(i - m') k v^T,
+    n likewise with k alone, o = S^T q / (max(|n . q|, exp(-m')) + ``den_eps``). Each head's o over its root mean
+    square (eps, no gain of its own), the heads together times a gain and sigmoid(Wg h), then the output projection.
+    S, n and m are float32 and start at zero."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    v_dim: int
+    gate_cap: float
+    eps: float
+    den_eps: float = 1e-6
+
+    def __post_init__(self):
+        if self.n_heads < 1 or not 1 <= self.head_dim <= 256 or self.v_dim < 1:
+            raise ValueError(f"matrix memory: {self.n_heads} heads of {self.head_dim} (1 to 256) and {self.v_dim}")
+        if not self.gate_cap > 0:
+            raise ValueError("gate_cap must be positive")
 
 
 @dataclass(frozen=True)

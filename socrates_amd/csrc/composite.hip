@@ -175,19 +175,20 @@ SOC_EXPORT int soc_depth_average(float* residual, float* kept, int count, const 
 // ---- biases, norms, rotation over interleaved pairs, turned values, page writes -------------------------------
 // x: rows of ld elements that hold, from col_q / col_k / col_v on, Hq heads of D, Hkv heads of D and Hkv heads of
 // Dv; bias (or null): float32 [ld], added to those columns. norm 0: none; 1: q and k RMS-normed per head with gains
-// [D]; 2: over the whole of q (gain [Hq D]) and the whole of k (gain [Hkv D]). Then elements 2i and 2i + 1 of the
-// first 2 * half of every q and k head are turned by position * inv_freq[i], and (value_freq given) elements 2m and
+// [D]; 2: over the whole of q (gain [Hq D]) and the whole of k (gain [Hkv D]); 3: per head behind the rotation, no
+// gain. Then elements 2i and 2i + 1 of the
+// first 2 * half of every q and k head are turned by position * inv_freq[i] (cosines and sines times magnitude), and (value_freq given) elements 2m and
 // 2m + 1 of every v head by position * value_freq[m]. q goes to q_out [N, Hq, P], k and v to the token's place in the
-// pools [pages, Hkv, BS, P] (P even), zeros behind D and Dv. grid (tokens, groups of per heads); a workgroup's q and k
-// heads pass through LDS (dynamic, per * D floats).
+// pools [pages, Hkv, BS, P] (P even), zeros behind D and Dv (Hkv 0: queries only, no pools). grid (tokens, groups of
+// per heads); a workgroup's q and k heads pass through LDS (dynamic, per * D floats).
 template <typename T>
 __global__ void __launch_bounds__(256)
 window_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int col_v, const float* __restrict__ bias,
                       T* __restrict__ q_out, T* __restrict__ k_pool, T* __restrict__ v_pool, const int* __restrict__ table,
                       int table_width, const int* __restrict__ token_rows, const int* __restrict__ positions,
                       const float* __restrict__ q_gain, const float* __restrict__ k_gain, int norm, float eps,
-                      const float* __restrict__ inv_freq, int half, const float* __restrict__ value_freq, int Hq, int Hkv,
-                      int D, int Dv, int P, int BS, int per) {
+                      const float* __restrict__ inv_freq, int half, float magnitude, const float* __restrict__ value_freq,
+                      int Hq, int Hkv, int D, int Dv, int P, int BS, int per) {
     extern __shared__ float qk[];                          // the workgroup's heads: [per][D]
     __shared__ float scratch[16];
     const int n = blockIdx.x, tid = threadIdx.x;
@@ -229,7 +230,31 @@ window_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int
         }
         __syncthreads();
     }
-    const int page = table[(size_t)token_rows[n] * table_width + pos / BS];
+    if (norm == 3) {
+        // turned in place, then each head over its root mean square; the writes below then turn nothing
+        for (int e = tid; e < (h_hi - h_lo) * half; e += 256) {
+            float* head = qk + (size_t)(e / half) * D;
+            const int j = e % half;
+            float sn, cs;
+            sincosf((float)pos * inv_freq[j], &sn, &cs);
+            sn *= magnitude; cs *= magnitude;
+            const float a = head[2 * j], b = head[2 * j + 1];
+            head[2 * j] = a * cs - b * sn;
+            head[2 * j + 1] = b * cs + a * sn;
+        }
+        __syncthreads();
+        const int wave = tid / SOC_WAVE, lane = tid % SOC_WAVE;
+        for (int h = h_lo + wave; h < h_hi; h += 256 / SOC_WAVE) {
+            float* head = qk + (size_t)(h - h_lo) * D;
+            float ss = 0.f;
+            for (int i = lane; i < D; i += SOC_WAVE) ss = fmaf(head[i], head[i], ss);
+            const float inv = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+            for (int i = lane; i < D; i += SOC_WAVE) head[i] = head[i] * inv;
+        }
+        __syncthreads();
+        half = 0;
+    }
+    const int page = Hkv ? table[(size_t)token_rows[n] * table_width + pos / BS] : 0;
     const size_t place = (size_t)page * Hkv * BS + (size_t)(pos % BS);
     // A thread owns one pair (2j, 2j + 1) of the padded head size and walks heads with it: the pair's angle is taken
     // once (P is even: the pools' head size; 256 / (P / 2) threads share a pair's heads among them).
@@ -237,7 +262,7 @@ window_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int
     const int j = tid % PP, g = tid / PP;
     if (g < lanes) {
         float sn = 0.f, cs = 1.f;
-        if (j < half) sincosf((float)pos * inv_freq[j], &sn, &cs);
+        if (j < half) { sincosf((float)pos * inv_freq[j], &sn, &cs); sn *= magnitude; cs *= magnitude; }
         for (int h = h_lo + g; h < h_hi; h += lanes) {
             const float* head = qk + (size_t)(h - h_lo) * D;
             const float a = 2 * j < D ? head[2 * j] : 0.f, b = 2 * j + 1 < D ? head[2 * j + 1] : 0.f;
@@ -263,12 +288,13 @@ window_prepare_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, int
 SOC_EXPORT int soc_window_prepare(const void* x, int ld, int col_q, int col_k, int col_v, const float* bias, void* q_out,
                                   void* k_pool, void* v_pool, const int* table, int table_width, const int* token_rows,
                                   const int* positions, const float* q_gain, const float* k_gain, int norm, float eps,
-                                  const float* inv_freq, int half, const float* value_freq, int N, int Hq, int Hkv, int D,
-                                  int Dv, int P, int BS, int dtype, hipStream_t stream) {
+                                  const float* inv_freq, int half, float magnitude, const float* value_freq, int N, int Hq,
+                                  int Hkv, int D, int Dv, int P, int BS, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (D < 1 || Dv < 1 || D > P || Dv > P || P > 256 || P % 2 || 2 * half > D || BS < 1 || norm < 0 || norm > 2 || Hq < 1 || Hkv < 1)
+    if (D < 1 || Dv < 1 || D > P || Dv > P || P > 256 || P % 2 || 2 * half > D || BS < 1 || norm < 0 || norm > 3 || Hq < 1 || Hkv < 0)
         return (int)hipErrorInvalidValue;
-    if (norm && (!q_gain || !k_gain)) return (int)hipErrorInvalidValue;
+    if (Hkv > 0 && (!k_pool || !v_pool || !table)) return (int)hipErrorInvalidValue;
+    if ((norm == 1 || norm == 2) && (!q_gain || !k_gain)) return (int)hipErrorInvalidValue;
     if (half && !inv_freq) return (int)hipErrorInvalidValue;
     if (value_freq && Dv % 2) return (int)hipErrorInvalidValue;
     // A token's heads go to as many workgroups as give the step about two per compute unit (a decode step has few
@@ -285,7 +311,7 @@ SOC_EXPORT int soc_window_prepare(const void* x, int ld, int col_q, int col_k, i
 #define SOC_WP(T)                                                                                                             \
     hipLaunchKernelGGL(window_prepare_kernel<T>, dim3(N, groups), dim3(256), lds, stream, (const T*)x, ld, col_q, col_k,       \
                        col_v, bias, (T*)q_out, (T*)k_pool, (T*)v_pool, table, table_width, token_rows, positions, q_gain,      \
-                       k_gain, norm, eps, inv_freq, half, value_freq, Hq, Hkv, D, Dv, P, BS, per)
+                       k_gain, norm, eps, inv_freq, half, magnitude, value_freq, Hq, Hkv, D, Dv, P, BS, per)
     if (dtype == 0) SOC_WP(float); else SOC_WP(bf16);
 #undef SOC_WP
     return soc_last_error();
@@ -415,7 +441,9 @@ __global__ void linear_prepare_kernel(const T* __restrict__ x, int ld, int col_q
 // x: rows of ld elements with H heads of D (q, from col_q; k, from col_k) and H heads of Dv (v, from col_v); with
 // act they pass silu; q is scaled by q_scale. CHANNEL: the decay of token t, head h, key channel i is
 // exp(logsigmoid(z[t, h D + i] + z_bias[h D + i]) / tau), z float32; else decays[h]. The state [H, D, Dv] of the
-// sequence's row is float32; a workgroup owns CW columns of one head, thread (part, column) a slice of the keys;
+// sequence's row is float32. prepared: prep [N, 3, H D] (q, k, decay per token, head and key channel, float32) comes
+// filled from the caller and nothing else of q and k is read. ones: the last ``ones`` of the Dv value columns are
+// not in x (whose heads hold Dv - ones) and read 1. A workgroup owns CW columns of one head, thread (part, column) a slice of the keys;
 // tokens go in batches staged through LDS with the next batch's loads in flight. o: float32 [N, H * Dv].
 template <typename T, int DK, int CW, bool CHANNEL>
 __global__ void __launch_bounds__(256)
@@ -423,7 +451,7 @@ linear_attention_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, i
                         const float* __restrict__ decays, const float* __restrict__ z, const float* __restrict__ z_bias,
                         float inv_tau, int H, int D, int Dv, float* __restrict__ state, size_t stride, int offset,
                         const int* __restrict__ seq_qstart, const int* __restrict__ seq_rows, const float* __restrict__ prep,
-                        float* __restrict__ out) {
+                        int ones, float* __restrict__ out) {
     constexpr int REC_TB = rec_batch(DK), PARTS = 256 / CW, KPT = DK / PARTS, STAGE = (REC_TB * DK + 255) / 256;
     __shared__ float sq[2][REC_TB][DK], sk[2][REC_TB][DK];
     __shared__ float sa[CHANNEL ? 2 : 1][CHANNEL ? REC_TB : 1][CHANNEL ? DK : 1];
@@ -472,7 +500,8 @@ linear_attention_kernel(const T* __restrict__ x, int ld, int col_q, int col_k, i
         }
 #pragma unroll
         for (int t = 0; t < REC_TB; ++t) {
-            float v = (live && n0 + t < hi) ? to_float(x[(size_t)(n0 + t) * ld + col_v + head * Dv + col]) : 0.f;
+            const int held = Dv - ones;
+            float v = (live && n0 + t < hi) ? (col < held ? to_float(x[(size_t)(n0 + t) * ld + col_v + head * held + col]) : 1.f) : 0.f;
             fv[t] = act ? cmp_silu(v) : v;
         }
     };
@@ -535,12 +564,12 @@ template <typename T, int DK>
 static void launch_linear_attention(const void* x, int ld, int col_q, int col_k, int col_v, float q_scale, int act,
                                     const float* decays, const float* z, const float* z_bias, float inv_tau, int H, int D, int Dv,
                                     float* state, long long stride, int offset, const int* seq_qstart, const int* seq_rows,
-                                    const float* prep, float* out, int n_seqs, int cw, hipStream_t stream) {
+                                    const float* prep, int prepared, int ones, float* out, int n_seqs, int cw, hipStream_t stream) {
 #define SOC_LA_LAUNCH(CW, CH)                                                                                                  \
     hipLaunchKernelGGL((linear_attention_kernel<T, DK, CW, CH>), dim3(H * ((Dv + CW - 1) / CW), n_seqs), dim3(256), 0, stream, \
                        (const T*)x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state,        \
-                       (size_t)stride, offset, seq_qstart, seq_rows, prep, out)
-    if (z) { if (cw == 16) SOC_LA_LAUNCH(16, true); else SOC_LA_LAUNCH(64, true); }
+                       (size_t)stride, offset, seq_qstart, seq_rows, prep, ones, out)
+    if (z || prepared) { if (cw == 16) SOC_LA_LAUNCH(16, true); else SOC_LA_LAUNCH(64, true); }
     else   { if (cw == 16) SOC_LA_LAUNCH(16, false); else SOC_LA_LAUNCH(64, false); }
 #undef SOC_LA_LAUNCH
 }
@@ -548,14 +577,15 @@ static void launch_linear_attention(const void* x, int ld, int col_q, int col_k,
 SOC_EXPORT int soc_linear_attention(const void* x, int ld, int col_q, int col_k, int col_v, float q_scale, int act,
                                     const float* decays, const float* z, const float* z_bias, float tau, int H, int D, int Dv,
                                     float* state, long long stride, int offset, const int* seq_qstart, const int* seq_rows,
-                                    float* prep, int n_tokens, float* out, int n_seqs, int max_q_len, int dtype,
-                                    hipStream_t stream) {
+                                    float* prep, int prepared, int ones, int n_tokens, float* out, int n_seqs, int max_q_len,
+                                    int dtype, hipStream_t stream) {
     if (n_seqs <= 0 || H <= 0) return 0;
-    if (D < 1 || D > 256 || Dv < 1 || n_seqs > 65535) return (int)hipErrorInvalidValue;
-    if ((z == nullptr) == (decays == nullptr) || (z && (!z_bias || !(tau > 0.f)))) return (int)hipErrorInvalidValue;
+    if (D < 1 || D > 256 || Dv < 1 || n_seqs > 65535 || ones < 0 || ones >= Dv) return (int)hipErrorInvalidValue;
+    if (prepared ? (!prep || z || decays)
+                 : ((z == nullptr) == (decays == nullptr) || (z && (!z_bias || !(tau > 0.f))))) return (int)hipErrorInvalidValue;
     const int cw = columns_per_workgroup(H, Dv, n_seqs, max_q_len);
     const float inv_tau = z ? 1.f / tau : 0.f;
-    if (prep) {                                            // scratch [n_tokens, 2 or 3, H * D]
+    if (prep && !prepared) {                                            // scratch [n_tokens, 2 or 3, H * D]
         if (n_tokens <= 0) return (int)hipErrorInvalidValue;
         const size_t total = (size_t)n_tokens * H * D;
         const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
@@ -566,8 +596,8 @@ SOC_EXPORT int soc_linear_attention(const void* x, int ld, int col_q, int col_k,
             hipLaunchKernelGGL(linear_prepare_kernel<bf16>, dim3(blocks), dim3(256), 0, stream, (const bf16*)x, ld, col_q, col_k,
                                q_scale, act, z, z_bias, inv_tau, H * D, total, prep);
     }
-#define SOC_LA_F32(DK) launch_linear_attention<float, DK>(x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, prep, out, n_seqs, cw, stream)
-#define SOC_LA_BF16(DK) launch_linear_attention<bf16, DK>(x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, prep, out, n_seqs, cw, stream)
+#define SOC_LA_F32(DK) launch_linear_attention<float, DK>(x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, prep, prepared, ones, out, n_seqs, cw, stream)
+#define SOC_LA_BF16(DK) launch_linear_attention<bf16, DK>(x, ld, col_q, col_k, col_v, q_scale, act, decays, z, z_bias, inv_tau, H, D, Dv, state, stride, offset, seq_qstart, seq_rows, prep, prepared, ones, out, n_seqs, cw, stream)
     if (dtype == 0) { SOC_BY_STATE_SIZE(D, SOC_LA_F32) } else { SOC_BY_STATE_SIZE(D, SOC_LA_BF16) }
     return soc_last_error();
 }

@@ -344,8 +344,9 @@ SOC_EXPORT int soc_relu_squared(const void* x, void* out, long long total, int d
 }
 
 // ---- the choice of experts ----------------------------------------------------------------------------------
-// One wave per token. s = softmax(z) over E experts (E <= 256); choice scores c = s + correction (if given).
-// Experts lie in n_groups equal groups of neighbours; a group's score is its largest c; only experts of the
+// One wave per token. s = softmax(z) over E experts (E <= 256), or sigmoid(z) each; z rows are ldz apart; choice
+// scores c = s + correction (if given). Experts lie in n_groups equal groups of neighbours; a group's score is the
+// sum of its group_top largest c (1: its largest); the weights are multiplied by scale; only experts of the
 // keep_groups best groups can be chosen (n_groups <= 1: all). The top experts by c (the lower index among
 // equals) are chosen; their weights are their s over the sum of the chosen s (+ renorm_eps).
 __device__ __forceinline__ void wave_argmax(float& v, int& i) {
@@ -358,8 +359,9 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 }
 
 __global__ void __launch_bounds__(256)
-moe_route_kernel(const float* __restrict__ z, const float* __restrict__ correction, int N, int E, int top, int n_groups,
-                 int keep_groups, float renorm_eps, int* __restrict__ idx, float* __restrict__ weight) {
+moe_route_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ correction, int N, int E, int top, int n_groups,
+                 int keep_groups, float renorm_eps, int sigmoid, int group_top, float scale, int* __restrict__ idx,
+                 float* __restrict__ weight) {
     __shared__ float sc[4][256];
     __shared__ float ss[4][256];
     const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE;
@@ -369,17 +371,18 @@ moe_route_kernel(const float* __restrict__ z, const float* __restrict__ correcti
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int e = lane + j * SOC_WAVE;
-        zv[j] = e < E ? z[(size_t)n * E + e] : -INFINITY;
+        zv[j] = e < E ? z[(size_t)n * ldz + e] : -INFINITY;
         m = fmaxf(m, zv[j]);
     }
     m = wave_max(m);
     float sum = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        zv[j] = lane + j * SOC_WAVE < E ? expf(zv[j] - m) : 0.f;
+        if (sigmoid) zv[j] = lane + j * SOC_WAVE < E ? hyb_sigmoid(zv[j]) : 0.f;
+        else zv[j] = lane + j * SOC_WAVE < E ? expf(zv[j] - m) : 0.f;
         sum += zv[j];
     }
-    sum = wave_sum(sum);
+    sum = sigmoid ? 1.f : wave_sum(sum);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int e = lane + j * SOC_WAVE;
@@ -398,8 +401,26 @@ moe_route_kernel(const float* __restrict__ z, const float* __restrict__ correcti
         for (int j = 0; j < 4; ++j) {
             const int g = lane + j * SOC_WAVE;
             gs[j] = -INFINITY;
-            if (g < n_groups)
+            if (g < n_groups && group_top <= 1)
                 for (int e = g * per; e < (g + 1) * per; ++e) gs[j] = fmaxf(gs[j], sc[wave][e]);
+            if (g < n_groups && group_top > 1) {
+                // the group_top largest, one after the other: each the largest that comes behind the last one
+                // taken in the order (score falling, index rising)
+                float pv = INFINITY, acc = 0.f;
+                int pi = -1;
+                for (int r = 0; r < group_top && r < per; ++r) {
+                    float bv = -INFINITY;
+                    int bi = -1;
+                    for (int e = g * per; e < (g + 1) * per; ++e) {
+                        const float v = sc[wave][e];
+                        const bool behind = v < pv || (v == pv && e > pi);
+                        if (behind && (bi < 0 || v > bv)) { bv = v; bi = e; }
+                    }
+                    if (bi < 0) break;
+                    acc += bv; pv = bv; pi = bi;
+                }
+                gs[j] = acc;
+            }
         }
         bool kept[4] = {false, false, false, false};
         for (int r = 0; r < keep_groups; ++r) {
@@ -446,17 +467,18 @@ moe_route_kernel(const float* __restrict__ z, const float* __restrict__ correcti
         if (lane == 0) { idx[(size_t)n * top + r] = bi; sc[wave][r] = ss[wave][bi]; }     // (sc is free: cv holds it)
     }
     if (lane == 0)
-        for (int r = 0; r < top; ++r) weight[(size_t)n * top + r] = sc[wave][r] / (total + renorm_eps);
+        for (int r = 0; r < top; ++r) weight[(size_t)n * top + r] = sc[wave][r] / (total + renorm_eps) * scale;
 }
 
-SOC_EXPORT int soc_moe_route(const float* z, const float* correction, int N, int E, int top, int n_groups, int keep_groups,
-                             float renorm_eps, int* idx, float* weight, hipStream_t stream) {
+SOC_EXPORT int soc_moe_route(const float* z, int ldz, const float* correction, int N, int E, int top, int n_groups, int keep_groups,
+                             float renorm_eps, int sigmoid, int group_top, float scale, int* idx, float* weight,
+                             hipStream_t stream) {
     if (N <= 0) return 0;
-    if (E < 1 || E > 256 || top < 1 || top > E || n_groups < 1 || E % n_groups || keep_groups < 1 || keep_groups > n_groups ||
+    if (E < 1 || E > 256 || ldz < E || group_top < 1 || top < 1 || top > E || n_groups < 1 || E % n_groups || keep_groups < 1 || keep_groups > n_groups ||
         (long long)keep_groups * (E / n_groups) < top)
         return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL(moe_route_kernel, dim3((N + 3) / 4), dim3(256), 0, stream, z, correction, N, E, top, n_groups, keep_groups,
-                       renorm_eps, idx, weight);
+    hipLaunchKernelGGL(moe_route_kernel, dim3((N + 3) / 4), dim3(256), 0, stream, z, ldz, correction, N, E, top, n_groups,
+                       keep_groups, renorm_eps, sigmoid, group_top, scale, idx, weight);
     return soc_last_error();
 }
 
@@ -520,13 +542,13 @@ SOC_EXPORT int soc_moe_sort(const int* idx, int M, int E, int TM, int max_tiles,
 // out[p, o] = sum_k x[src(p), k] w[e, o, k] for the places p of expert e's run, o < n_out. src(p) = pair_at[p] / top
 // (rows of x are tokens) if pair_at is given, else p (rows of x are places). A workgroup takes one tile of 16
 // places x 64 outputs, 32 k at a time through LDS; float32 sums, k in order. With ff > 0 the weights hold
-// [gate (ff) | up (ff)] rows and the kernel writes act[p, o] = g sigmoid(slope g) (u + 1), g = min(gate, limit),
+// [gate (ff) | up (ff)] rows and the kernel writes act[p, o] = g sigmoid(slope g) (u + shift), g = min(gate, limit),
 // u = clamp(up, -limit, limit), o < ff, from both products.
 template <typename T, typename TO, bool GLU>
 __global__ void __launch_bounds__(256)
 grouped_linear_kernel(const T* __restrict__ x, int ldx, const int* __restrict__ pair_at, int top, const T* __restrict__ w,
                       const int* __restrict__ offsets, const int* __restrict__ tiles, TO* __restrict__ out, int n_out, int K,
-                      int ff, float limit, float slope) {
+                      int ff, float limit, float slope, float shift) {
     __shared__ float xs[16][33], ws[64][33], wu[GLU ? 64 : 1][33];
     __shared__ int rows[16];
     const int e = tiles[2 * blockIdx.y];
@@ -575,7 +597,7 @@ grouped_linear_kernel(const T* __restrict__ x, int ldx, const int* __restrict__ 
                 // gate and up are rounded as the compute dtype stores them before the activation
                 const float g = fminf(to_float(from_float<T>(acc[t])), limit);
                 const float u = fminf(fmaxf(to_float(from_float<T>(acu[t])), -limit), limit);
-                y = g * hyb_sigmoid(slope * g) * (u + 1.f);
+                y = g * hyb_sigmoid(slope * g) * (u + shift);
             }
             out[(size_t)p * n_out + o0 + to] = from_float<TO>(y);
         }
@@ -594,7 +616,7 @@ template <int WM, int WN, int MI, int NI, bool GLU, typename TO>
 __global__ void __launch_bounds__(256)
 grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__ pair_at, int top, const bf16* __restrict__ w,
                     const int* __restrict__ offsets, const int* __restrict__ tiles, TO* __restrict__ out, int n_out, int K, int ff,
-                    float limit, float slope) {
+                    float limit, float slope, float shift) {
     constexpr int BM = WM * MI * 16, BN = WN * NI * 16, COLS = GLU ? BN / 2 : BN;
     constexpr int A_PER = (BM * 8 + 255) / 256, W_PER = BN * 8 / 256;
     static_assert(WM * WN == 4 && (!GLU || NI % 2 == 0), "four waves; gate and up tiles in pairs");
@@ -708,7 +730,7 @@ grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__
                     if (col >= ff) continue;
                     const float g = fminf(to_float(from_float<bf16>(acc[i][j][r])), limit);
                     const float u = fminf(fmaxf(to_float(from_float<bf16>(acc[i][j + 1][r])), -limit), limit);
-                    out[(size_t)p * n_out + col] = from_float<TO>(g * hyb_sigmoid(slope * g) * (u + 1.f));
+                    out[(size_t)p * n_out + col] = from_float<TO>(g * hyb_sigmoid(slope * g) * (u + shift));
                 }
             } else {
 #pragma unroll
@@ -725,7 +747,7 @@ grouped_mfma_kernel(const bf16* __restrict__ x, int ldx, const int* __restrict__
 // matrix cores) or 128 (bfloat16 on the matrix cores only).
 SOC_EXPORT int soc_grouped_linear(const void* x, int ldx, const int* pair_at, int top, const void* w, const int* offsets,
                                   const int* tiles, int max_tiles, int tile, void* out, int n_out, int K, int ff, float limit,
-                                  float slope, int out_f32, int dtype, hipStream_t stream) {
+                                  float slope, float shift, int out_f32, int dtype, hipStream_t stream) {
     if (max_tiles <= 0 || n_out <= 0) return 0;
     if (K < 1 || max_tiles > 65535 || (ff > 0 && (ff != n_out || out_f32))) return (int)hipErrorInvalidValue;
     const bool mfma = dtype == 1 && K % 8 == 0 && ldx % 8 == 0;
@@ -734,7 +756,7 @@ SOC_EXPORT int soc_grouped_linear(const void* x, int ldx, const int* pair_at, in
 #define SOC_GM(WM, WN, MI, NI, GLU, TO)                                                                                          \
     hipLaunchKernelGGL((grouped_mfma_kernel<WM, WN, MI, NI, GLU, TO>), dim3((n_out + (GLU ? 63 : 127)) / (GLU ? 64 : 128), max_tiles), \
                        dim3(256), 0, stream, (const bf16*)x, ldx, pair_at, top, (const bf16*)w, offsets, tiles, (TO*)out, n_out, \
-                       K, ff, limit, slope)
+                       K, ff, limit, slope, shift)
         if (tile == 128) {
             if (ff > 0) SOC_GM(2, 2, 4, 4, true, bf16); else if (out_f32) SOC_GM(2, 2, 4, 4, false, float); else SOC_GM(2, 2, 4, 4, false, bf16);
         } else {
@@ -746,7 +768,7 @@ SOC_EXPORT int soc_grouped_linear(const void* x, int ldx, const int* pair_at, in
     const dim3 grid((n_out + 63) / 64, max_tiles);
 #define SOC_GL(T, TO, GLU)                                                                                                    \
     hipLaunchKernelGGL((grouped_linear_kernel<T, TO, GLU>), grid, dim3(256), 0, stream, (const T*)x, ldx, pair_at, top,       \
-                       (const T*)w, offsets, tiles, (TO*)out, n_out, K, ff, limit, slope)
+                       (const T*)w, offsets, tiles, (TO*)out, n_out, K, ff, limit, slope, shift)
     if (ff > 0) { if (dtype == 0) SOC_GL(float, float, true); else SOC_GL(bf16, bf16, true); }
     else if (dtype == 0) SOC_GL(float, float, false);
     else if (out_f32) SOC_GL(bf16, float, false);
@@ -756,28 +778,31 @@ SOC_EXPORT int soc_grouped_linear(const void* x, int ldx, const int* pair_at, in
 }
 
 // ---- the weighted sum of a token's experts ---------------------------------------------------------------------------
-// out[n, c] = sum_r weight[n, r] y[place[n top + r], c] (+ extra[n, c]), float32; y float32 [M, d] by place.
+// out[n, c] = sum_r weight[n, r] y[place[n top + r], c] (+ extra[n, c], times sigmoid(gate[n ldg]) if gate is given), float32;
+// y float32 [M, d] by place.
 template <typename T>
 __global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ place, const float* __restrict__ weight,
-                                   const T* __restrict__ extra, float* __restrict__ out, int N, int d, int top) {
+                                   const T* __restrict__ extra, const float* __restrict__ gate, int ldg, float* __restrict__ out,
+                                   int N, int d, int top) {
     const int n = blockIdx.y;
+    const float open = (extra && gate) ? hyb_sigmoid(gate[(size_t)n * ldg]) : 1.f;
     for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < d; c += gridDim.x * blockDim.x) {
-        float acc = extra ? to_float(extra[(size_t)n * d + c]) : 0.f;
+        float acc = extra ? open * to_float(extra[(size_t)n * d + c]) : 0.f;
         for (int r = 0; r < top; ++r)
             acc = fmaf(weight[(size_t)n * top + r], y[(size_t)place[(size_t)n * top + r] * d + c], acc);
         out[(size_t)n * d + c] = acc;
     }
 }
 
-SOC_EXPORT int soc_moe_combine(const float* y, const int* place, const float* weight, const void* extra, float* out, int N, int d,
-                               int top, int dtype, hipStream_t stream) {
+SOC_EXPORT int soc_moe_combine(const float* y, const int* place, const float* weight, const void* extra, const float* gate, int ldg,
+                               float* out, int N, int d, int top, int dtype, hipStream_t stream) {
     if (N <= 0 || d <= 0) return 0;
     if (N > 65535) return (int)hipErrorInvalidValue;
     const dim3 grid((d + 255) / 256 < 16 ? (d + 255) / 256 : 16, N);
     if (dtype == 0)
-        hipLaunchKernelGGL(moe_combine_kernel<float>, grid, dim3(256), 0, stream, y, place, weight, (const float*)extra, out, N, d, top);
+        hipLaunchKernelGGL(moe_combine_kernel<float>, grid, dim3(256), 0, stream, y, place, weight, (const float*)extra, gate, ldg, out, N, d, top);
     else
-        hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, dim3(256), 0, stream, y, place, weight, (const bf16*)extra, out, N, d, top);
+        hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, dim3(256), 0, stream, y, place, weight, (const bf16*)extra, gate, ldg, out, N, d, top);
     return soc_last_error();
 }
 

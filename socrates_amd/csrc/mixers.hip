@@ -29,17 +29,25 @@ __device__ __forceinline__ void store8(bf16* p, const float (&x)[8]) {
 // ---- the close of a branch ---------------------------------------------------------------------
 // residual += mult * gain * g / rms(g) with g = y * sigmoid(logits + bias) (no gate: g = y); the logits are the
 // first d elements of rows of ldg elements (they may be columns of a wider product);
-// then, if next_gain is given, out = residual / rms(residual) * next_gain.
+// then, if next_gain is given, out = residual / rms(residual) * next_gain. y is in the compute dtype, or float32 if
+// y_f32; y_bias (float32 [d], or null) is added to it first.
+template <typename T>
+__device__ __forceinline__ float branch_result(const void* y, int y_f32, const float* y_bias, size_t at, int c) {
+    const float v = y_f32 ? ((const float*)y)[at] : to_float(((const T*)y)[at]);
+    return y_bias ? v + y_bias[c] : v;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
-gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits, int ldg,
+gated_norm_add_kernel(float* __restrict__ residual, const void* __restrict__ y, int y_f32, const float* __restrict__ y_bias,
+                      const T* __restrict__ logits, int ldg,
                       const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
                       const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
     __shared__ float scratch[16];
     const size_t base = (size_t)blockIdx.x * d, gbase = (size_t)blockIdx.x * ldg;
     float ss = 0.f;
     for (int c = threadIdx.x; c < d; c += blockDim.x) {
-        float g = to_float(y[base + c]);
+        float g = branch_result<T>(y, y_f32, y_bias, base + c, c);
         if (logits) g *= soc_sigmoid(to_float(logits[gbase + c]) + bias[c]);
         ss += g * g;
     }
@@ -47,7 +55,7 @@ gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, con
     const float scale = mult / sqrtf(ss / (float)d + eps);
     float rr = 0.f;
     for (int c = threadIdx.x; c < d; c += blockDim.x) {
-        float g = to_float(y[base + c]);
+        float g = branch_result<T>(y, y_f32, y_bias, base + c, c);
         if (logits) g *= soc_sigmoid(to_float(logits[gbase + c]) + bias[c]);
         const float r = residual[base + c] + scale * gain[c] * g;
         residual[base + c] = r;
@@ -64,7 +72,8 @@ gated_norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y, con
 // read once, all loads are issued before the first is used.
 template <typename T, int PER>
 __global__ void __launch_bounds__(256)
-gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits, int ldg,
+gated_norm_add_regs_kernel(float* __restrict__ residual, const void* __restrict__ y, int y_f32, const float* __restrict__ y_bias,
+                           const T* __restrict__ logits, int ldg,
                            const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
                            const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
     __shared__ float scratch[16];
@@ -74,7 +83,7 @@ gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y
     for (int i = 0; i < PER; ++i) {
         const int c = threadIdx.x + i * 256;
         const bool in = c < d;
-        g[i] = in ? to_float(y[base + c]) : 0.f;
+        g[i] = in ? branch_result<T>(y, y_f32, y_bias, base + c, c) : 0.f;
         gate[i] = (in && logits) ? to_float(logits[gbase + c]) + bias[c] : 0.f;
         res[i] = in ? residual[base + c] : 0.f;
         gn[i] = in ? gain[c] : 0.f;
@@ -115,7 +124,8 @@ gated_norm_add_regs_kernel(float* __restrict__ residual, const T* __restrict__ y
 // the first loads, so the kernel waits for memory once.
 template <typename T, int CH>
 __global__ void __launch_bounds__(256)
-gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y, const T* __restrict__ logits, int ldg,
+gated_norm_add_vec8_kernel(float* __restrict__ residual, const void* __restrict__ y, int y_f32, const float* __restrict__ y_bias,
+                           const T* __restrict__ logits, int ldg,
                            const float* __restrict__ bias, const float* __restrict__ gain, float eps, float mult,
                            const float* __restrict__ next_gain, float next_eps, T* __restrict__ out, int d) {
     __shared__ float scratch[16];
@@ -125,7 +135,14 @@ gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y
     for (int i = 0; i < CH; ++i) {
         const int c = (threadIdx.x + i * 256) * 8;
         if (c < d) {
-            VecLoad<T, 8>::load(y + base + c, g[i]);
+            if (y_f32) VecLoad<float, 8>::load((const float*)y + base + c, g[i]);
+            else VecLoad<T, 8>::load((const T*)y + base + c, g[i]);
+            if (y_bias) {
+                float yb[8];
+                VecLoad<float, 8>::load(y_bias + c, yb);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) g[i][e] += yb[e];
+            }
             VecLoad<float, 8>::load(residual + base + c, res[i]);
             VecLoad<float, 8>::load(gain + c, gn[i]);
             if (logits) {
@@ -175,17 +192,18 @@ gated_norm_add_vec8_kernel(float* __restrict__ residual, const T* __restrict__ y
 }
 
 template <typename T>
-static void launch_gated_norm_add(float* residual, const void* y, const void* logits, int ldg, const float* bias, const float* gain,
+static void launch_gated_norm_add(float* residual, const void* y, int y_f32, const float* y_bias, const void* logits, int ldg, const float* bias, const float* gain,
                                   float eps, float mult, const float* next_gain, float next_eps, void* out, int N, int d,
                                   hipStream_t stream) {
 #define SOC_GNA(PER)                                                                                                    \
-    hipLaunchKernelGGL((gated_norm_add_regs_kernel<T, PER>), dim3(N), dim3(256), 0, stream, residual, (const T*)y,     \
+    hipLaunchKernelGGL((gated_norm_add_regs_kernel<T, PER>), dim3(N), dim3(256), 0, stream, residual, y, y_f32, y_bias, \
                        (const T*)logits, ldg, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
 #define SOC_GNA8(CH)                                                                                                    \
-    hipLaunchKernelGGL((gated_norm_add_vec8_kernel<T, CH>), dim3(N), dim3(256), 0, stream, residual, (const T*)y,      \
+    hipLaunchKernelGGL((gated_norm_add_vec8_kernel<T, CH>), dim3(N), dim3(256), 0, stream, residual, y, y_f32, y_bias,  \
                        (const T*)logits, ldg, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d)
     // (pieces of eight elements: the width, the logits' rows and their first element all sit at multiples of 8)
-    const bool by8 = d % 8 == 0 && ldg % 8 == 0 && ((uintptr_t)logits % (8 * sizeof(T))) == 0;
+    const bool by8 = d % 8 == 0 && ldg % 8 == 0 && ((uintptr_t)logits % (8 * sizeof(T))) == 0 &&
+                     ((uintptr_t)y % (y_f32 ? 32 : 8 * sizeof(T))) == 0;
     if (by8 && d <= 2048) SOC_GNA8(1);
     else if (by8 && d <= 4096) SOC_GNA8(2);
     else if (by8 && d <= 8192) SOC_GNA8(4);
@@ -194,16 +212,16 @@ static void launch_gated_norm_add(float* residual, const void* y, const void* lo
     else if (d <= 4096) SOC_GNA(16);
     else if (d <= 8192) SOC_GNA(32);
     else
-        hipLaunchKernelGGL(gated_norm_add_kernel<T>, dim3(N), dim3(256), 0, stream, residual, (const T*)y, (const T*)logits,
+        hipLaunchKernelGGL(gated_norm_add_kernel<T>, dim3(N), dim3(256), 0, stream, residual, y, y_f32, y_bias, (const T*)logits,
                            ldg, bias, gain, eps, mult, next_gain, next_eps, (T*)out, d);
 }
 
-SOC_EXPORT int soc_gated_norm_add(float* residual, const void* y, const void* logits, int ldg, const float* bias,
+SOC_EXPORT int soc_gated_norm_add(float* residual, const void* y, int y_f32, const float* y_bias, const void* logits, int ldg, const float* bias,
                                   const float* gain, float eps, float mult, const float* next_gain, float next_eps,
                                   void* out, int N, int d, int dtype, hipStream_t stream) {
     if (N <= 0) return 0;
-    if (dtype == 0) launch_gated_norm_add<float>(residual, y, logits, ldg, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
-    else launch_gated_norm_add<bf16>(residual, y, logits, ldg, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
+    if (dtype == 0) launch_gated_norm_add<float>(residual, y, y_f32, y_bias, logits, ldg, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
+    else launch_gated_norm_add<bf16>(residual, y, y_f32, y_bias, logits, ldg, bias, gain, eps, mult, next_gain, next_eps, out, N, d, stream);
     return soc_last_error();
 }
 

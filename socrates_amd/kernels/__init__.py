@@ -12,7 +12,8 @@ norms, sampling); ``products.py`` the matrix products in all their forms, ``atte
 attention and what prepares it, ``planning.py`` the host arithmetic of key splits,
 ``mixers.py`` the mixers with a state per row, attention over a cached latent and blocks with norms
 on both sides of a branch, ``hybrid.py`` attention whose keys and values differ in size, retention, routed
-experts and a per-token side input, ``common.py`` what they share, ``build.py`` the compiler and loader.
+experts and a per-token side input, ``memory.py`` a matrix memory with exponential gates and the two maps of
+differential attention, ``common.py`` what they share, ``build.py`` the compiler and loader.
 """
 
 from __future__ import annotations
@@ -25,6 +26,7 @@ import torch
 from .attention import Attention
 from .composite import Composite
 from .hybrid import Hybrid
+from .memory import Memory
 from .mixers import Mixers
 from .build import KernelBuildError, build_all, compile_library, load_library
 from .common import (_ATTENTION_SIGNATURES, _DTYPE_CODE, _EW_SIGNATURES, _GEMM_SIGNATURES, _SAMPLING_SIGNATURES, KernelError,
@@ -36,7 +38,7 @@ __all__ = ["HipKernels", "KernelBuildError", "KernelError", "MAX_KEY_SPLITS", "N
            "compile_library", "load_library", "plan_key_splits"]
 
 
-class HipKernels(Products, Attention, Mixers, Hybrid, Composite):
+class HipKernels(Products, Attention, Mixers, Hybrid, Composite, Memory):
     def __init__(self, dtype=torch.bfloat16, device="cuda:0"):
         if dtype not in _DTYPE_CODE:
             raise ValueError(f"compute dtype must be float32 or bfloat16, not {dtype}")

@@ -52,7 +52,7 @@ _GEMM_SIGNATURES = {
 }
 L = c_longlong
 _MIXER_SIGNATURES = {
-    "soc_gated_norm_add": [P, P, P, I, P, P, F, F, P, F, P, I, I, I, P],
+    "soc_gated_norm_add": [P, P, I, P, P, I, P, P, F, F, P, F, P, I, I, I, P],
     "soc_glu_clamped": [P, P, I, I, I, F, F, I, P],
     "soc_token_shift": [P, P, I, P, L, I, P, P, P, I, I, I, I, I, P],
     "soc_wkv_decay": [P, P, P, P, I, I, I, I, P],
@@ -70,10 +70,10 @@ _HYBRID_SIGNATURES = {
     "soc_head_gate": [P, P, I, P, I, I, I, I, I, P],
     "soc_retention": [P, I, I, I, I, P, P, I, F, P, I, I, I, P, L, I, P, P, P, I, P, I, I, I, P],
     "soc_relu_squared": [P, P, L, I, P],
-    "soc_moe_route": [P, P, I, I, I, I, I, F, P, P, P],
+    "soc_moe_route": [P, I, P, I, I, I, I, I, F, I, I, F, P, P, P],
     "soc_moe_sort": [P, I, I, I, I, P, P, P, P, P],
-    "soc_grouped_linear": [P, I, P, I, P, P, P, I, I, P, I, I, I, F, F, I, I, P],
-    "soc_moe_combine": [P, P, P, P, P, I, I, I, I, P],
+    "soc_grouped_linear": [P, I, P, I, P, P, P, I, I, P, I, I, I, F, F, F, I, I, P],
+    "soc_moe_combine": [P, P, P, P, P, I, P, I, I, I, I, P],
     "soc_side_gate": [P, P, I, I, P, I, P, I, I, I, P],
     "soc_add_cast": [P, P, P, I, L, P, I, P],
 }
@@ -81,12 +81,17 @@ _COMPOSITE_SIGNATURES = {
     "soc_norm_add_cast": [P, P, I, P, F, P, I, I, P, I, P, I, P],
     "soc_depth_begin": [P, P, P, L, I, P],
     "soc_depth_average": [P, P, I, P, P, L, I, P],
-    "soc_window_prepare": [P, I, I, I, I, P, P, P, P, P, I, P, P, P, P, I, F, P, I, P, I, I, I, I, I, I, I, I, P],
+    "soc_window_prepare": [P, I, I, I, I, P, P, P, P, P, I, P, P, P, P, I, F, P, I, F, P, I, I, I, I, I, I, I, I, P],
     "soc_pool_blocks": [P, P, P, I, P, P, P, I, P, P, P, I, I, I, I, I, I, I, P],
     "soc_turn_back": [P, P, P, P, I, I, I, I, I, P],
-    "soc_linear_attention": [P, I, I, I, I, F, I, P, P, P, F, I, I, I, P, L, I, P, P, P, I, P, I, I, I, P],
+    "soc_linear_attention": [P, I, I, I, I, F, I, P, P, P, F, I, I, I, P, L, I, P, P, P, I, I, I, P, I, I, I, P],
     "soc_scaled_sum": [P, I, F, P, I, F, P, P, I, I, I, P],
     "soc_glu_gelu": [P, P, I, I, I, I, P],
+}
+_MEMORY_SIGNATURES = {
+    "soc_memory_gates": [P, P, F, P, I, I, I, F, I, I, P, L, I, P, P, I, I, P, P, P, P, I, P],
+    "soc_memory_finish": [P, P, P, I, P, I, I, I, F, F, P, I, P],
+    "soc_diff_combine": [P, P, I, I, I, I, I, F, F, F, I, P],
 }
 _SAMPLING_SIGNATURES = {"soc_sample": [P, P, P, P, P, I, I, P], "soc_argmax": [P, P, P, I, I, I, P]}
 _ATTENTION_SIGNATURES = {

@@ -14,7 +14,7 @@ import torch
 from .build import load_library
 from .common import _COMPOSITE_SIGNATURES, KernelError, _check, _declare, _ptr
 
-_NORMS = {None: 0, "head": 1, "whole": 2}
+_NORMS = {None: 0, "head": 1, "whole": 2, "turned": 3}
 
 
 class Composite:
@@ -78,11 +78,13 @@ class Composite:
 
     # -- window attention ------------------------------------------------------------------------------------------
     def window_prepare(self, x, cols, Hq, Hkv, D, Dv, P, bias, q_gain, k_gain, norm, eps, inv_freq, rotary_dim, value_freq,
-                       positions, token_rows, slot):
+                       positions, token_rows, slot, magnitude=1.0):
         """x [N, ld] holds, from columns ``cols`` = (q, k, v) on, Hq heads of D, Hkv heads of D and Hkv heads of Dv;
         ``bias`` (float32 [ld] or None) is added to them. ``norm`` "head": q and k RMS-normed per head (gains [D]);
-        "whole": over the whole of q and of k (gains [Hq D], [Hkv D]); None: as they are. Pairs (2i, 2i + 1) of the
-        first ``rotary_dim`` elements of every q and k head are turned by position * inv_freq[i]; with ``value_freq``
+        "whole": over the whole of q and of k (gains [Hq D], [Hkv D]); "turned": per head behind the rotation, without
+        gains; None: as they are. Pairs (2i, 2i + 1) of the first ``rotary_dim`` elements of every q and k head are
+        turned by position * inv_freq[i], cosines and sines times ``magnitude``; ``slot`` None with Hkv 0: queries
+        only, nothing is written; with ``value_freq``
         [Dv / 2] the pairs of every v head by position * value_freq[m]. Keys and values go to the token's place in the
         pools [pages, Hkv, block, P], zeros behind D and Dv. Returns q [N, Hq, P], zeros behind D."""
         N, ld = x.shape
@@ -96,7 +98,7 @@ class Composite:
             raise KernelError(f"norm {norm!r}: head, whole or None")
         if bias is not None:
             self._want(bias, "bias", torch.float32, (ld,))
-        if norm is not None:
+        if norm in ("head", "whole"):
             self._want(q_gain, "q gain", torch.float32, (D,) if norm == "head" else (Hq * D,))
             self._want(k_gain, "k gain", torch.float32, (D,) if norm == "head" else (Hkv * D,))
         half = rotary_dim // 2
@@ -108,14 +110,21 @@ class Composite:
             self._want(value_freq, "value frequencies", torch.float32, (Dv // 2,))
         self._want(positions, "positions", torch.int32, (N,))
         self._want(token_rows, "token_rows", torch.int32, (N,))
-        self._check_slot(slot, Hkv, P)
+        if (slot is None) != (Hkv == 0):
+            raise KernelError("queries alone come with no kv heads and no cache slot")
+        gains = norm in ("head", "whole")
+        if slot is None:
+            kp, vp, table, width, bs = None, None, None, 0, 1
+        else:
+            self._check_slot(slot, Hkv, P)
+            kp, vp, table, width, bs = slot.k, slot.v, slot.block_table, slot.block_table.shape[1], slot.block_size
         q = torch.empty((N, Hq, P), dtype=self.dtype, device=self.device)
         _check(self._composite().soc_window_prepare(
-            _ptr(x), c_int(ld), c_int(col_q), c_int(col_k), c_int(col_v), _ptr(bias), _ptr(q), _ptr(slot.k), _ptr(slot.v),
-            _ptr(slot.block_table), c_int(slot.block_table.shape[1]), _ptr(token_rows), _ptr(positions),
-            _ptr(q_gain if norm else None), _ptr(k_gain if norm else None), c_int(_NORMS[norm]), c_float(eps),
-            _ptr(inv_freq if half else None), c_int(half), _ptr(value_freq), c_int(N), c_int(Hq), c_int(Hkv), c_int(D), c_int(Dv),
-            c_int(P), c_int(slot.block_size), c_int(self.code), self._stream()), "window_prepare")
+            _ptr(x), c_int(ld), c_int(col_q), c_int(col_k), c_int(col_v), _ptr(bias), _ptr(q), _ptr(kp), _ptr(vp),
+            _ptr(table), c_int(width), _ptr(token_rows), _ptr(positions),
+            _ptr(q_gain if gains else None), _ptr(k_gain if gains else None), c_int(_NORMS[norm]), c_float(eps),
+            _ptr(inv_freq if half else None), c_int(half), c_float(magnitude), _ptr(value_freq), c_int(N), c_int(Hq), c_int(Hkv),
+            c_int(D), c_int(Dv), c_int(P), c_int(bs), c_int(self.code), self._stream()), "window_prepare")
         return q
 
     def pool_blocks(self, slot, ctx):
@@ -154,40 +163,50 @@ class Composite:
         return out
 
     # -- linear attention ----------------------------------------------------------------------------------------
-    def linear_attention(self, x, cols, H, D, Dv, q_scale, activate, decays, z, z_bias, tau, state, offset, ctx):
+    def linear_attention(self, x, cols, H, D, Dv, q_scale, activate, decays, z, z_bias, tau, state, offset, ctx,
+                         prepared=None, ones=0):
         """S <- diag(decay) S + k v^T, o = S^T q per head over each sequence's tokens, from and into the row's state
         ([H, D, Dv] from ``offset``). x [N, ld] holds q and k (H heads of D) and v (H heads of Dv) from columns
         ``cols`` on; with ``activate`` they pass silu; q is scaled by ``q_scale``. The decay is ``decays`` [H], or, with
-        ``z`` (float32 [N, H D]), sigmoid(z + z_bias)^(1 / tau) per token and key channel. float32 [N, H * Dv]."""
+        ``z`` (float32 [N, H D]), sigmoid(z + z_bias)^(1 / tau) per token and key channel. float32 [N, H * Dv].
+        ``prepared`` (float32 [N, 3, H D]): q, k and the decays per token, head and key channel as the caller made them
+        (x then gives the values only). ``ones``: the last that many of the Dv value columns are not in x, whose heads
+        hold Dv - ones, and read 1 (a sum of the keys beside the state)."""
         N, ld = x.shape
         self._want(x, "x", self.dtype)
         col_q, col_k, col_v = cols
-        if min(cols) < 0 or max(col_q, col_k) + H * D > ld or col_v + H * Dv > ld:
+        if not 0 <= ones < Dv:
+            raise KernelError(f"{ones} columns of ones among {Dv}")
+        if min(cols) < 0 or max(col_q, col_k) + H * D > ld or col_v + H * (Dv - ones) > ld:
             raise KernelError(f"queries, keys and values from columns {cols} do not fit rows of {ld}")
         if not 1 <= D <= 256 or Dv < 1:
             raise KernelError(f"linear attention: heads of {D} and {Dv}")
-        if (z is None) == (decays is None):
+        if prepared is not None:
+            if z is not None or decays is not None or activate:
+                raise KernelError("linear attention: prepared q, k and decays come alone")
+            self._want(prepared, "prepared q, k and decays", torch.float32, (N, 3, H * D))
+        elif (z is None) == (decays is None):
             raise KernelError("linear attention: a decay per head, or per token and key channel")
         if z is not None:
             self._want(z, "decay logits", torch.float32, (N, H * D))
             self._want(z_bias, "decay bias", torch.float32, (H * D,))
             if not tau > 0:
                 raise KernelError("tau is positive")
-        else:
+        elif prepared is None:
             self._want(decays, "decays", torch.float32, (H,))
         stride = self._state(state, offset, H * D * Dv, ctx)
         out = torch.empty((N, H * Dv), dtype=torch.float32, device=self.device)
         # a step with a portion of some length: activations, the scale and the decays are taken once, ahead of the
         # walk (each of a head's workgroups would take them again); single tokens and short portions where they
         # are staged
-        prep = None
-        if (activate or z is not None) and ctx.max_q_len >= self.linear_prepare_ahead:
+        prep = prepared
+        if prepared is None and (activate or z is not None) and ctx.max_q_len >= self.linear_prepare_ahead:
             prep = torch.empty((N, 3 if z is not None else 2, H * D), dtype=torch.float32, device=self.device)
         _check(self._composite().soc_linear_attention(
             _ptr(x), c_int(ld), c_int(col_q), c_int(col_k), c_int(col_v), c_float(q_scale), c_int(1 if activate else 0),
             _ptr(decays), _ptr(z), _ptr(z_bias), c_float(tau), c_int(H), c_int(D), c_int(Dv), _ptr(state), stride, c_int(offset),
-            _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), _ptr(prep), c_int(N), _ptr(out), c_int(ctx.n_seqs), c_int(ctx.max_q_len),
-            c_int(self.code), self._stream()), "linear_attention")
+            _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), _ptr(prep), c_int(1 if prepared is not None else 0), c_int(ones), c_int(N),
+            _ptr(out), c_int(ctx.n_seqs), c_int(ctx.max_q_len), c_int(self.code), self._stream()), "linear_attention")
         return out
 
     # -- sums and activations ----------------------------------------------------------------------------------------

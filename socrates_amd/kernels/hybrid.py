@@ -146,12 +146,19 @@ class Hybrid:
                "relu_squared")
         return out
 
-    def moe_route(self, logits, correction, top, n_groups=1, keep_groups=1, renorm_eps=1e-20):
-        """logits float32 [N, E]: scores are their softmax; the choice goes by score + correction among the
-        experts of the ``keep_groups`` best of ``n_groups`` equal groups of neighbours (a group's score is its best
-        choice score). Returns (experts int32 [N, top], weights float32 [N, top]: the chosen scores over their sum)."""
+    def moe_route(self, logits, correction, top, n_groups=1, keep_groups=1, renorm_eps=1e-20, scoring="softmax", group_top=1,
+                  scale=1.0):
+        """logits float32 [N, E] (they may be columns of a wider product): scores are their softmax, or with ``scoring``
+        "sigmoid" the sigmoid of each; the choice goes by score + correction among the experts of the ``keep_groups``
+        best of ``n_groups`` equal groups of neighbours (a group's score is the sum of its ``group_top`` best choice
+        scores). Returns (experts int32 [N, top], weights float32 [N, top]: the chosen scores over their sum, times
+        ``scale``)."""
         N, E = logits.shape
-        self._want(logits, "router logits", torch.float32)
+        if (logits.device.type != "cuda" or logits.dtype != torch.float32 or logits.stride(1) != 1
+                or (N > 1 and logits.stride(0) < E)):
+            raise KernelError(f"router logits {tuple(logits.shape)} {logits.dtype} with strides {logits.stride()}")
+        if scoring not in ("softmax", "sigmoid") or group_top < 1:
+            raise KernelError(f"routing: scoring {scoring!r}, groups scored by their {group_top} best")
         if correction is not None:
             self._want(correction, "correction", torch.float32, (E,))
         if (not 1 <= E <= MAX_EXPERTS or not 1 <= top <= E or n_groups < 1 or E % n_groups or not 1 <= keep_groups <= n_groups
@@ -159,8 +166,10 @@ class Hybrid:
             raise KernelError(f"routing: {top} of {E} experts (at most {MAX_EXPERTS}) from {keep_groups} of {n_groups} groups")
         idx = torch.empty((N, top), dtype=torch.int32, device=self.device)
         weight = torch.empty((N, top), dtype=torch.float32, device=self.device)
-        _check(self._hybrid().soc_moe_route(_ptr(logits), _ptr(correction), c_int(N), c_int(E), c_int(top), c_int(n_groups),
-                                            c_int(keep_groups), c_float(renorm_eps), _ptr(idx), _ptr(weight), self._stream()),
+        _check(self._hybrid().soc_moe_route(_ptr(logits), c_int(logits.stride(0) if N > 1 else E), _ptr(correction), c_int(N), c_int(E),
+                                            c_int(top), c_int(n_groups), c_int(keep_groups), c_float(renorm_eps),
+                                            c_int(1 if scoring == "sigmoid" else 0), c_int(group_top), c_float(scale), _ptr(idx),
+                                            _ptr(weight), self._stream()),
                "moe_route")
         return idx, weight
 
@@ -184,8 +193,9 @@ class Hybrid:
 
     def grouped_linear(self, x, w, runs, by_token, glu=None, out_dtype=None):
         """out[p] = w[e] x[row of p] for every place p of expert e's run; x rows are tokens (``by_token``: place p
-        reads the token of its pair) or places. w [E, n_out, K]; with ``glu`` = (limit, slope) w holds [gate | up]
-        rows and out [M, n_out / 2] is g sigmoid(slope g) (u + 1) with g = min(gate, limit), u = clamp(up, +-limit)."""
+        reads the token of its pair) or places. w [E, n_out, K]; with ``glu`` = (limit, slope[, shift = 1]) w holds
+        [gate | up] rows and out [M, n_out / 2] is g sigmoid(slope g) (u + shift) with g = min(gate, limit),
+        u = clamp(up, +-limit)."""
         self._want(x, "x", self.dtype)
         self._want(w, "weights per expert", self.dtype)
         M = runs.place.numel()
@@ -202,35 +212,45 @@ class Hybrid:
         if out_dtype not in (self.dtype, torch.float32) or (glu is not None and out_dtype != self.dtype):
             raise KernelError(f"products per expert: a result in {out_dtype}")
         out = torch.empty((M, n_out), dtype=out_dtype, device=self.device)
-        limit, slope = glu if glu is not None else (0.0, 0.0)
+        limit, slope, shift = (tuple(glu) + (1.0,))[:3] if glu is not None else (0.0, 0.0, 1.0)
         _check(self._hybrid().soc_grouped_linear(
             _ptr(x), c_int(x.stride(0)), _ptr(runs.pair_at if by_token else None), c_int(runs.top), _ptr(w), _ptr(runs.offsets),
             _ptr(runs.tiles), c_int(runs.tiles.shape[0]), c_int(runs.tile), _ptr(out), c_int(n_out), c_int(K), c_int(ff), c_float(limit),
-            c_float(slope), c_int(1 if out_dtype == torch.float32 and self.dtype != torch.float32 else 0), c_int(self.code),
+            c_float(slope), c_float(shift), c_int(1 if out_dtype == torch.float32 and self.dtype != torch.float32 else 0), c_int(self.code),
             self._stream()), "grouped_linear")
         return out
 
-    def moe_combine(self, y, runs, weight, extra=None):
+    def moe_combine(self, y, runs, weight, extra=None, extra_gate=None):
         """float32 [N, d]: each token's weighted sum of its experts' rows of ``y`` (float32 [M, d] by place), plus
-        ``extra`` [N, d] (compute dtype) if given."""
+        ``extra`` [N, d] (compute dtype) if given, times sigmoid(``extra_gate``) (float32 [N], which may be a column
+        of a wider product) if that is given."""
         N, top = weight.shape
         d = y.shape[1]
         self._want(y, "expert results", torch.float32, (N * top, d))
         self._want(weight, "weights", torch.float32)
         if extra is not None:
             self._want(extra, "extra", self.dtype, (N, d))
+        ldg = 0
+        if extra_gate is not None:
+            if (extra is None or extra_gate.device.type != "cuda" or extra_gate.dtype != torch.float32
+                    or tuple(extra_gate.shape) != (N,)):
+                raise KernelError("the gate of the extra term: float32 [N] beside an extra term")
+            ldg = extra_gate.stride(0) if N > 1 else 1
         out = torch.empty((N, d), dtype=torch.float32, device=self.device)
         step = 65535
         for lo in range(0, N, step):
             n = min(step, N - lo)
             _check(self._hybrid().soc_moe_combine(_ptr(y), _ptr(runs.place[lo * top:]), _ptr(weight[lo:]),
-                                                  _ptr(extra[lo:]) if extra is not None else None, _ptr(out[lo:]), c_int(n), c_int(d),
+                                                  _ptr(extra[lo:]) if extra is not None else None,
+                                                  _ptr(extra_gate[lo:]) if extra_gate is not None else None, c_int(ldg),
+                                                  _ptr(out[lo:]), c_int(n), c_int(d),
                                                   c_int(top), c_int(self.code), self._stream()), "moe_combine")
         return out
 
-    def moe_experts(self, x, idx, weight, w_gate_up, w_down, limit, slope, extra=None):
-        """The weighted sum of each token's chosen experts (clamped gated feed-forwards: ``w_gate_up`` [E, 2 ff, d],
-        ``w_down`` [E, d, ff]) plus ``extra``; float32 [N, d]."""
+    def moe_experts(self, x, idx, weight, w_gate_up, w_down, limit, slope, extra=None, shift=1.0, extra_gate=None):
+        """The weighted sum of each token's chosen experts (gated feed-forwards with the activation
+        g sigmoid(slope g) (u + shift) under a clamp: ``w_gate_up`` [E, 2 ff, d], ``w_down`` [E, d, ff]) plus ``extra``
+        (times sigmoid(``extra_gate``) per token if given); float32 [N, d]."""
         E, _, d = w_gate_up.shape
         ff = w_down.shape[2]
         # many tokens per expert, in bfloat16 with rows that start on 16 bytes: the larger tiles of the matrix cores
@@ -239,9 +259,9 @@ class Hybrid:
         if self.dtype == torch.bfloat16 and d % 8 == 0 and ff % 8 == 0 and x.stride(0) % 8 == 0:
             tile = next((t for least, t in EXPERT_TILES_MANY if idx.numel() >= least * E), EXPERT_TILE)
         runs = self.moe_sort(idx, E, tile)
-        act = self.grouped_linear(x, w_gate_up, runs, by_token=True, glu=(limit, slope))
+        act = self.grouped_linear(x, w_gate_up, runs, by_token=True, glu=(limit, slope, shift))
         y = self.grouped_linear(act, w_down, runs, by_token=False, out_dtype=torch.float32)
-        return self.moe_combine(y, runs, weight, extra)
+        return self.moe_combine(y, runs, weight, extra, extra_gate)
 
     # -- a per-token side input, and the residual sum with a cast -----------------------------------------------------
     def side_gate(self, t, table, col0, token_ids):

@@ -21,14 +21,19 @@ class Mixers:
         return lib
 
     # -- blocks ----------------------------------------------------------------------------------
-    def gated_norm_add(self, residual, y, gate_logits, gate_bias, gain, eps, mult, next_gain=None, next_eps=0.0):
+    def gated_norm_add(self, residual, y, gate_logits, gate_bias, gain, eps, mult, next_gain=None, next_eps=0.0, y_bias=None):
         """residual (float32 [N, d], in place) += mult * gain * g / rms(g) with g = y *
         sigmoid(gate_logits + gate_bias) (no gate: g = y). With ``next_gain``: returns
         residual / rms(residual) * next_gain in the compute dtype; else None. ``gate_logits`` may be
-        [N, d] columns of a wider product (rows apart by its width)."""
+        [N, d] columns of a wider product (rows apart by its width). ``y`` is in the compute dtype or float32;
+        ``y_bias`` (float32 [d]) is added to it first."""
         N, d = residual.shape
         self._want(residual, "residual", torch.float32)
-        self._want(y, "branch result", self.dtype, (N, d))
+        if y.dtype not in (self.dtype, torch.float32):
+            raise KernelError(f"a branch's result in {y.dtype}")
+        self._want(y, "branch result", y.dtype, (N, d))
+        if y_bias is not None:
+            self._want(y_bias, "the result's bias", torch.float32, (d,))
         self._want(gain, "norm gain", torch.float32, (d,))
         ldg = 0
         if gate_logits is not None:
@@ -42,7 +47,7 @@ class Mixers:
             self._want(next_gain, "next norm's gain", torch.float32, (d,))
             out = torch.empty((N, d), dtype=self.dtype, device=self.device)
         _check(self._mixers().soc_gated_norm_add(
-            _ptr(residual), _ptr(y), _ptr(gate_logits), c_int(ldg), _ptr(gate_bias if gate_logits is not None else None), _ptr(gain),
+            _ptr(residual), _ptr(y), c_int(1 if y.dtype == torch.float32 else 0), _ptr(y_bias), _ptr(gate_logits), c_int(ldg), _ptr(gate_bias if gate_logits is not None else None), _ptr(gain),
             c_float(eps), c_float(mult), _ptr(next_gain), c_float(next_eps), _ptr(out), c_int(N), c_int(d),
             c_int(self.code), self._stream()), "gated_norm_add")
         return out

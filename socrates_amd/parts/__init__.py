@@ -1,5 +1,5 @@
-from . import (attention, block, feedforward, gated_attention, latent_attention, linear_attention, norm, parallel,  # noqa: F401
-               recurrent, retention, rope, routed, side, window_attention)  # noqa: F401  (registers the parts)
+from . import (attention, block, differential_attention, feedforward, gated_attention, latent_attention,  # noqa: F401
+               linear_attention, matrix_memory, norm, parallel, recurrent, retention, rope, routed, side, window_attention)  # noqa: F401  (registers the parts)
 from .block import build_block, register_arrangement
 from .model import DecoderModel, cache_needs, expected_tensors
 from .registry import (PagedKV, PagedLatent, RowState, TensorDecl, build_part, impl_of, register_part,

@@ -63,6 +63,15 @@ class Normed:
         self.rows = rows
 
 
+class Biased:
+    """What a branch returns when its last product's bias is left to whoever adds the result: ``rows`` (float32 or
+    the compute dtype) and ``bias`` (float32 [d])."""
+    __slots__ = ("rows", "bias")
+
+    def __init__(self, rows, bias):
+        self.rows, self.bias = rows, bias
+
+
 class PreNormBlock:
     chains = True       # forward takes ``nxt``, the block that runs after this one
 
@@ -159,10 +168,15 @@ class SandwichBlock:
             (y, logits), bias = y, gate.bias
         elif gate is not None:
             logits, bias = ops.linear(h, gate.weight), gate.bias
+        more = {}
+        if isinstance(y, Biased):                       # the result's own bias, added before the norm
+            y, more["y_bias"] = y.rows, y.bias
+        if y.dim() == 3 and y.shape[0] == 1:            # float32 sums of a feed-forward that sums in float32
+            y = y[0]
         gain, eps = post_norm.fusable()
         follows = next_norm.fusable() if hasattr(next_norm, "fusable") else None
         out = ops.gated_norm_add(residual, y, logits, bias, gain, eps, self.spec.residual_mult,
-                                 *(follows or (None, 0.0)))
+                                 *(follows or (None, 0.0)), **more)
         if next_norm is not None and follows is None:
             out = next_norm.add_norm(residual, None)
         return out

@@ -12,16 +12,17 @@ from .registry import TensorDecl, register_part
 class SwiGLU:
     @staticmethod
     def tensors(spec: SwiGLUSpec):
-        return {"gate_proj.weight": TensorDecl((spec.intermediate, spec.hidden)),
-                "up_proj.weight": TensorDecl((spec.intermediate, spec.hidden)),
-                "down_proj.weight": TensorDecl((spec.hidden, spec.intermediate))}
+        gate, up, down = spec.names
+        return {gate: TensorDecl((spec.intermediate, spec.hidden)),
+                up: TensorDecl((spec.intermediate, spec.hidden)),
+                down: TensorDecl((spec.hidden, spec.intermediate))}
 
     def __init__(self, spec: SwiGLUSpec, tensors, ops):
         self.spec, self.ops = spec, ops
         # One operand for gate and up. Where the width allows, their rows alternate in blocks
         # of 16 (16 gate rows, the 16 up rows of the same columns, ...): a workgroup of the
         # decode product then holds both and applies the activation itself.
-        gate, up = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        gate, up = tensors[spec.names[0]], tensors[spec.names[1]]
         ff = spec.intermediate
         self.interleave = 16 if ff % 16 == 0 else 0
         if self.interleave:
@@ -29,7 +30,7 @@ class SwiGLU:
                                          dim=1).reshape(2 * ff, -1).contiguous()
         else:
             self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
-        self.w_down = tensors["down_proj.weight"]
+        self.w_down = tensors[spec.names[2]]
         # (the activation goes to a product and nowhere else: the kernel set may lay it out as it likes)
         self._free_layout = {"by_tile": True} if getattr(ops, "rows_by_tile", None) is not None else {}
 

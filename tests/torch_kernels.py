@@ -174,8 +174,10 @@ class TorchKernels:
         return out
 
     # -- what closes a branch of a block with norms on both sides ------------------------------
-    def gated_norm_add(self, residual, y, gate_logits, gate_bias, gain, eps, mult, next_gain=None, next_eps=0.0):
+    def gated_norm_add(self, residual, y, gate_logits, gate_bias, gain, eps, mult, next_gain=None, next_eps=0.0, y_bias=None):
         y = y.to(self.acc)
+        if y_bias is not None:
+            y = y + y_bias.to(self.acc)
         if gate_logits is not None:
             y = y * torch.sigmoid(gate_logits.to(self.acc) + gate_bias.to(self.acc))
         residual += (mult * self._norm(y, gain, eps)).to(residual.dtype)
@@ -183,11 +185,11 @@ class TorchKernels:
             return None
         return self._norm(residual, next_gain, next_eps).to(self.dtype)
 
-    def glu_clamped(self, gate_up, limit, slope, ff=None):
+    def glu_clamped(self, gate_up, limit, slope, ff=None, shift=1.0):
         ff = ff or gate_up.shape[-1] // 2
         g = torch.clamp(gate_up[..., :ff].to(self.acc), max=limit)
         u = torch.clamp(gate_up[..., ff:2 * ff].to(self.acc), min=-limit, max=limit)
-        return (g * torch.sigmoid(slope * g) * (u + 1)).to(self.dtype)
+        return (g * torch.sigmoid(slope * g) * (u + shift)).to(self.dtype)
 
     # -- mixers with a state per row -------------------------------------------------------------
     @staticmethod
@@ -274,12 +276,12 @@ class TorchKernels:
         return (y if gate_first else y * gate).to(self.dtype)
 
     # -- attention over a cached latent ------------------------------------------------------------
-    def _turn_pairs(self, x, positions, inv_freq):
+    def _turn_pairs(self, x, positions, inv_freq, magnitude=1.0):
         """Pairs (2i, 2i + 1) of the first 2 * len(inv_freq) elements of the last axis; x [N, ..., D]."""
         dims = 2 * inv_freq.numel()
         ang = positions.to(torch.float32)[:, None] * inv_freq.to(torch.float32)[None, :]
         shape = [x.shape[0]] + [1] * (x.dim() - 2) + [dims // 2]
-        cos, sin = ang.cos().to(self.acc).view(shape), ang.sin().to(self.acc).view(shape)
+        cos, sin = (ang.cos().to(self.acc) * magnitude).view(shape), (ang.sin().to(self.acc) * magnitude).view(shape)
         a, b = x[..., 0:dims:2], x[..., 1:dims:2]
         out = x.clone()
         out[..., 0:dims:2] = a * cos - b * sin
@@ -373,14 +375,15 @@ class TorchKernels:
     def relu_squared(self, x):
         return (torch.relu(x.to(self.acc)) ** 2).to(self.dtype)
 
-    def moe_route(self, logits, correction, top, n_groups=1, keep_groups=1, renorm_eps=1e-20):
+    def moe_route(self, logits, correction, top, n_groups=1, keep_groups=1, renorm_eps=1e-20, scoring="softmax",
+                  group_top=1, scale=1.0):
         A = self.acc
-        s = torch.softmax(logits.to(A), dim=-1)
+        s = torch.softmax(logits.to(A), dim=-1) if scoring == "softmax" else torch.sigmoid(logits.to(A))
         c = s if correction is None else s + correction.to(A)
         N, E = s.shape
         if n_groups > 1 and keep_groups < n_groups:
             per = E // n_groups
-            best = c.view(N, n_groups, per).max(-1).values
+            best = c.view(N, n_groups, per).sort(-1, descending=True).values[..., :group_top].sum(-1)
             kept = torch.zeros((N, n_groups), dtype=torch.bool, device=s.device)
             for _ in range(keep_groups):                      # the lower index among equals
                 g = torch.where(kept, torch.full_like(best, -float("inf")), best).argmax(-1)
@@ -396,20 +399,20 @@ class TorchKernels:
             idx[:, r] = first
             taken[torch.arange(N), first] = True
         w = torch.gather(s, 1, idx)
-        w = w / (w.sum(-1, keepdim=True) + renorm_eps)
+        w = w / (w.sum(-1, keepdim=True) + renorm_eps) * scale
         return idx.to(torch.int32), w.to(torch.float32 if A == torch.float32 else A)
 
-    def moe_experts(self, x, idx, weight, w_gate_up, w_down, limit, slope, extra=None):
+    def moe_experts(self, x, idx, weight, w_gate_up, w_down, limit, slope, extra=None, shift=1.0, extra_gate=None):
         A = self.acc
         N, top = idx.shape
         ff = w_gate_up.shape[1] // 2
         out = torch.zeros((N, w_down.shape[1]), dtype=A, device=x.device)
         if extra is not None:
-            out += extra.to(A)
+            out += extra.to(A) if extra_gate is None else extra.to(A) * torch.sigmoid(extra_gate.to(A)).unsqueeze(-1)
         for r in range(top):
             e = idx[:, r].long()
             both = torch.einsum("nk,nok->no", x.to(A), w_gate_up[e].to(A)).to(self.dtype)
-            act = self.glu_clamped(both, limit, slope, ff)
+            act = self.glu_clamped(both, limit, slope, ff, shift)
             y = torch.einsum("nk,nok->no", act.to(A), w_down[e].to(A))
             out += weight[:, r:r + 1].to(A) * y
         return out.to(torch.float32 if A == torch.float32 else A)
@@ -444,7 +447,7 @@ class TorchKernels:
         return residual.to(self.dtype) if cast else None
 
     def window_prepare(self, x, cols, Hq, Hkv, D, Dv, P, bias, q_gain, k_gain, norm, eps, inv_freq, rotary_dim, value_freq,
-                       positions, token_rows, slot):
+                       positions, token_rows, slot, magnitude=1.0):
         A = self.acc
         N = x.shape[0]
         cq, ck, cv = cols
@@ -458,12 +461,17 @@ class TorchKernels:
         if norm == "head":
             q, k = self._norm(q, q_gain, eps), self._norm(k, k_gain, eps)
         if rotary_dim:
-            q = self._turn_pairs(q, positions, inv_freq)
-            k = self._turn_pairs(k, positions, inv_freq)
+            q = self._turn_pairs(q, positions, inv_freq, magnitude)
+            k = self._turn_pairs(k, positions, inv_freq, magnitude)
+        if norm == "turned":
+            q = q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + eps)
+            k = k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + eps)
         if value_freq is not None:
             v = self._turn_pairs(v, positions, value_freq)
         out = torch.zeros((N, Hq, P), dtype=self.dtype, device=x.device)
         out[..., :D] = q.to(self.dtype)
+        if slot is None:
+            return out
         kp = torch.zeros((N, Hkv, P), dtype=slot.k.dtype, device=x.device)
         vp = torch.zeros((N, Hkv, P), dtype=slot.v.dtype, device=x.device)
         kp[..., :D] = k.to(slot.k.dtype)
@@ -493,17 +501,22 @@ class TorchKernels:
             y = self._turn_pairs(y, -positions, value_freq)
         return y.reshape(N, H * Dv).to(self.dtype)
 
-    def linear_attention(self, x, cols, H, D, Dv, q_scale, activate, decays, z, z_bias, tau, state, offset, ctx):
+    def linear_attention(self, x, cols, H, D, Dv, q_scale, activate, decays, z, z_bias, tau, state, offset, ctx,
+                         prepared=None, ones=0):
         A = self.acc
         N = x.shape[0]
         cq, ck, cv = cols
         q = x[:, cq:cq + H * D].reshape(N, H, D).to(A)
         k = x[:, ck:ck + H * D].reshape(N, H, D).to(A)
-        v = x[:, cv:cv + H * Dv].reshape(N, H, Dv).to(A)
+        v = x[:, cv:cv + H * (Dv - ones)].reshape(N, H, Dv - ones).to(A)
+        if ones:
+            v = torch.cat([v, torch.ones((N, H, ones), dtype=A, device=x.device)], dim=-1)
         if activate:
             q, k, v = q * torch.sigmoid(q), k * torch.sigmoid(k), v * torch.sigmoid(v)
         q = q * q_scale
-        if z is not None:
+        if prepared is not None:
+            q, k, decay = (prepared[:, j].reshape(N, H, D).to(A) for j in range(3))
+        elif z is not None:
             decay = torch.exp(torch.nn.functional.logsigmoid(z.to(A) + z_bias.to(A)) / tau).view(N, H, D)
         else:
             decay = decays.to(A).view(1, H, 1).expand(N, H, D)
@@ -515,6 +528,47 @@ class TorchKernels:
                 out[t] = torch.einsum("hk,hkv->hv", q[t], S)
             state[row, offset:offset + H * D * Dv] = S.reshape(-1).to(state.dtype)
         return out.reshape(N, H * Dv).to(torch.float32 if A == torch.float32 else A)
+
+    def memory_gates(self, gates, bias, cap, x, cols, H, D, q_scale, state, offset, ctx):
+        A = self.acc
+        N = x.shape[0]
+        cq, ck, _ = cols
+        g = cap * torch.tanh((gates.to(A) + bias.to(A)) / cap)
+        gi, gf = g[:, :H], torch.nn.functional.logsigmoid(g[:, H:])
+        q = x[:, cq:cq + H * D].reshape(N, H, D).to(A) * q_scale
+        k = x[:, ck:ck + H * D].reshape(N, H, D).to(A)
+        out_dtype = torch.float32 if A == torch.float32 else A
+        prep = torch.empty((N, 3, H * D), dtype=out_dtype, device=x.device)
+        maxima = torch.empty((N, H), dtype=out_dtype, device=x.device)
+        for row, lo, hi in self._sequences(ctx):
+            m = state[row, offset:offset + H].to(A).clone()
+            for t in range(lo, hi):
+                new = torch.maximum(gf[t] + m, gi[t])
+                prep[t, 0] = q[t].reshape(-1).to(out_dtype)
+                prep[t, 1] = (torch.exp(gi[t] - new).unsqueeze(-1) * k[t]).reshape(-1).to(out_dtype)
+                prep[t, 2] = torch.exp(gf[t] + m - new).unsqueeze(-1).expand(H, D).reshape(-1).to(out_dtype)
+                maxima[t] = new.to(out_dtype)
+                m = new
+            state[row, offset:offset + H] = m.to(state.dtype)
+        return prep, maxima
+
+    def memory_finish(self, raw, maxima, z, gain, H, Dv, eps, den_eps):
+        A = self.acc
+        N = raw.shape[0]
+        r = raw.view(N, H, Dv + 1).to(A)
+        den = torch.maximum(r[..., Dv].abs(), torch.exp(-maxima.to(A))) + den_eps
+        o = r[..., :Dv] / den.unsqueeze(-1)
+        o = o / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+        y = o.reshape(N, H * Dv) * gain.to(A) * torch.sigmoid(z[:, :H * Dv].to(A))
+        return y.to(self.dtype)
+
+    def diff_combine(self, o, H, G, P, Dv, lam, eps, out_scale):
+        A = self.acc
+        N = o.shape[0]
+        a = o.view(N, G, 2, H // G, P)[..., :Dv].to(A)
+        y = a[:, :, 0] - lam * a[:, :, 1]
+        y = y / torch.sqrt(y.pow(2).mean(-1, keepdim=True) + eps) * out_scale
+        return y.reshape(N, H * Dv).to(self.dtype)
 
     def scaled_sum(self, a, a_scale, b, b_scale, bias=None):
         y = a.to(self.acc)
