@@ -84,8 +84,8 @@ def softmax_attention(q, k, v, scale, ok, softcap=None):
     return out
 
 
-def mlstm(h, W, m, eps):
-    """Matrix memory with exponential gates held stable by a running maximum that starts at 0."""
+def mlstm(h, W, m, eps, first_max=0.0):
+    """Matrix memory with exponential gates held stable by a running maximum that starts at ``first_max`` (0)."""
     T = h.shape[0]
     H, D, Dv, cap = m["heads"], m["dim"], m["vdim"], float(m["gate_cap"])
     q = (h @ W["q"].T).view(T, H, D) * D ** -0.5
@@ -97,7 +97,7 @@ def mlstm(h, W, m, eps):
     for a in range(H):
         S = torch.zeros(D, Dv, dtype=F64)
         n = torch.zeros(D, dtype=F64)
-        mx = 0.0
+        mx = first_max
         for t in range(T):
             new = max(float(gf[t, a]) + mx, float(gi[t, a]))
             keep, take = math.exp(float(gf[t, a]) + mx - new), math.exp(float(gi[t, a]) - new)
@@ -185,8 +185,10 @@ def part(weights, prefix):
     return {k[len(prefix):]: v for k, v in weights.items() if k.startswith(prefix)}
 
 
-def forward(config, weights, tokens, residuals=None):
-    """Logits [T, vocab] of one sequence; ``residuals`` (a list) receives the stream after every layer."""
+def forward(config, weights, tokens, residuals=None, first_max=0.0):
+    """Logits [T, vocab] of one sequence; ``residuals`` (a list) receives the stream after every layer.
+    ``first_max``: where the running maxima of the matrix memories start (0 in the design; a test passes
+    another value to show that it would see the difference)."""
     W = {k: v.to(F64) for k, v in weights.items()}
     eps = float(config["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.long)
@@ -197,7 +199,7 @@ def forward(config, weights, tokens, residuals=None):
         p, m = f"l{i}.", layer["mixer"]
         h = rms(x, eps) * W[p + "norm1"]
         if layer["type"] == "mlstm":
-            y = mlstm(h, part(W, p + "mix."), m, eps)
+            y = mlstm(h, part(W, p + "mix."), m, eps, first_max)
         elif layer["type"] == "attention":
             y, kept[i] = differential_attention(h, part(W, p + "mix."), m, eps, positions,
                                                 kept[m["kv_from"]] if m.get("kv_from") is not None else None)
@@ -213,3 +215,14 @@ def forward(config, weights, tokens, residuals=None):
             residuals.append(x.clone())
     x = rms(x, eps) * W["final.norm"]
     return x @ W["embed"].T
+
+
+def greedy(config, weights, prompt, n_new):
+    """The n_new tokens that follow ``prompt`` when the largest logit is taken every time (the lowest index
+    among equals)."""
+    ids, out = list(prompt), []
+    for _ in range(n_new):
+        tok = int(forward(config, weights, ids)[-1].argmax())
+        out.append(tok)
+        ids.append(tok)
+    return out
