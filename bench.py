@@ -436,6 +436,81 @@ def pozalorn_beside_others(args, dtype, item):
     return 0
 
 
+def berelorn_dict(width, ff, n_layers, heads, kv_heads, window=1024):
+    """A Berelorn of ``n_layers`` layers at a real model's layer sizes, four kinds in turn: a matrix memory with
+    exponential gates (heads of 128 x 128), differential attention (two maps of 128 per head over values of 128, a
+    window that keeps the first four tokens, a ramp-stretched rotation), the same on the cache of the layer before
+    it, and causal attention whose values are its keys (heads of 128, soft-capped scores, a gate per head); every
+    feed-forward 32 silu-gated experts of a quarter of the dense size in four groups, four per token from two
+    groups by sigmoid scores, beside a gated shared one."""
+    rot = {"base": 1000000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    diff = {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "diff": 0.3,
+            "rot": rot, "mask": {"size": window, "keep_first": 4}}
+    keyed = {"heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "scale": 8.0, "softcap": 50.0,
+             "rot": dict(rot, dims=128)}
+    kinds = [{"type": "mlstm", "mixer": {"heads": width // 128, "dim": 128, "vdim": 128, "gate_cap": 15.0}},
+             {"type": "attention", "mixer": diff}, {"type": "attention", "mixer": dict(diff, kv_from=-1)},
+             {"type": "attention_2", "mixer": keyed}]
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "shared": {"ff": ff // 4},
+           "router": {"experts": 32, "top": 4, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+    layers = []
+    for i in range(n_layers):
+        layer = json.loads(json.dumps(kinds[i % 4]))
+        if layer["mixer"].get("kv_from") == -1:
+            layer["mixer"]["kv_from"] = i - 1
+        layer["mlp"] = json.loads(json.dumps(moe))
+        layers.append(layer)
+    return {"architecture": "Berelorn", "vocab": 151936, "width": width, "layers": layers, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 8.0}}
+
+
+def berelorn_beside_others(args, dtype, item):
+    """Prefill and decode of Berelorn at a few real layer sizes, beside Tedulorn (the closest model: attention over a
+    window with kept first tokens and a linear recurrence in turn, experts chosen among groups beside a shared one)
+    and Qwen3 of the same width, feed-forward size, vocabulary and number of layers, all with the library's default
+    solutions for its products. One JSON line of its own; the default workload and its line are untouched."""
+    import torch
+    sizes = [("4b", "qwen3-4b"), ("8b", "qwen3-8b")]
+    n_layers = args.layers or 12
+    out = {"metric": "prefill and decode of Berelorn beside Tedulorn and Qwen3 at equal width, feed-forward, vocabulary and layers",
+           "dtype": args.dtype, "layers": n_layers, "batch": args.batch, "context": args.context,
+           "prefill_tokens": args.prefill_tokens, "data": "synthetic: seeded random weights, uniform random token ids",
+           "sizes": {}}
+    only = set(filter(None, (args.only or "").split(",")))
+    for tag, preset in sizes:
+        if only & {name for name, _ in sizes} and tag not in only:
+            continue
+        q = preset_dict(preset)
+        q["num_hidden_layers"] = n_layers
+        t = tedulorn_dict(q["hidden_size"], q["intermediate_size"], n_layers, q["num_attention_heads"], q["num_key_value_heads"])
+        b = berelorn_dict(q["hidden_size"], q["intermediate_size"], n_layers, q["num_attention_heads"], q["num_key_value_heads"])
+        point = {}
+        for name, cfg in (("berelorn", b), ("tedulorn", t), ("qwen3", q)):
+            if only & {"berelorn", "tedulorn", "qwen3"} and name not in only:
+                continue
+            config, engine = build_engine(cfg, dtype, args.batch, args.max_len, seed=0, compile_=not args.no_graphs,
+                                          chunk=max(2048, args.prefill_tokens), block_size=args.block_size)
+            V = cfg.get("vocab_size") or cfg["vocab"]
+            tok_s, ms = decode_rate(engine, args.batch, args.context, args.steps, args.warmup, V, seed=1)
+            pre_s = prefill_rate(engine, args.prefill_tokens, V, seed=2)
+            if name == "qwen3":
+                weights = config.param_counts()["read_per_step"] * item
+                cache = args.batch * args.context * config.kv_bytes_per_token(item)
+            else:
+                weights = config.step_weight_bytes(args.batch, item)
+                cache = config.step_cache_bytes(args.batch, args.context, item)
+            point[name] = {"decode_tok_s": round(tok_s, 1), "decode_ms": round(ms, 4),
+                           "decode_hbm_frac": round((weights + cache) / (ms * 1e-3) / 1e9 / HBM_GBPS, 4),
+                           "prefill_ms": round(pre_s * 1e3, 3), "prefill_tok_s": round(args.prefill_tokens / pre_s, 1),
+                           "prefill_flop_frac": round(config.prefill_flops(args.prefill_tokens) / pre_s / PEAK_FLOPS[args.dtype], 4),
+                           "weights_gb": round(weights / 1e9, 3)}
+            release(engine)
+            torch.cuda.synchronize()
+        out["sizes"][tag] = point
+    print(json.dumps(out))
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -461,8 +536,12 @@ def main(argv=None):
     ap.add_argument("--pozalorn", action="store_true",
                     help="instead of the default workload: prefill and decode of Pozalorn at 4B- and 8B-sized layers "
                          "(--layers of them, default 12), each beside Tedulorn and Qwen3 of the same sizes")
+    ap.add_argument("--berelorn", action="store_true",
+                    help="instead of the default workload: prefill and decode of Berelorn at 4B- and 8B-sized layers "
+                         "(--layers of them, default 12), each beside Tedulorn and Qwen3 of the same sizes")
     ap.add_argument("--only", default=None,
-                    help="--tedulorn, --pozalorn: sizes and models to run, with commas (4b,8b,pozalorn,tedulorn,mitisun,qwen3)")
+                    help="--tedulorn, --pozalorn, --berelorn: sizes and models to run, with commas "
+                         "(4b,8b,berelorn,pozalorn,tedulorn,mitisun,qwen3)")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per page of the cache (the reference's 16)")
     ap.add_argument("--no-graphs", action="store_true")
@@ -496,6 +575,8 @@ def main(argv=None):
         return tedulorn_beside_others(args, dtype, item)
     if args.pozalorn:
         return pozalorn_beside_others(args, dtype, item)
+    if args.berelorn:
+        return berelorn_beside_others(args, dtype, item)
     if args.mixed:
         args.preset = args.preset or MIXED_PRESET
         args.max_len = max(args.max_len, 8192)
