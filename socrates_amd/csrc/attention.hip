@@ -414,6 +414,18 @@ struct FusedQkv {
     bf16* v_pool_w;
 };
 
+// A soft cap on the scores inside the kernels on the matrix cores: the raw score t becomes (cap / scale) tanh(t scale /
+// cap), so that what follows (the maximum, times scale log2 e) works on it as on a raw score. tanh(x) =
+// 1 - 2 / (exp2(2 x log2 e) + 1). ``a`` = cap / scale (0: no cap), ``b`` = 2 log2 e scale / cap.
+struct SoftCap {
+    float a, b;
+    __device__ __forceinline__ SoftCap(float scale, float cap)
+        : a(cap > 0.f ? cap / scale : 0.f), b(cap > 0.f ? 2.f * 1.44269504088896340736f * scale / cap : 0.f) {}
+    __device__ __forceinline__ float operator()(float t) const {
+        return a * (1.f - 2.f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(t * b) + 1.f));
+    }
+};
+
 template <int RT, bool TP, bool FUSED = false>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
@@ -423,7 +435,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                        int n_row_blocks, bf16* __restrict__ out, float* __restrict__ part_o,
                        float* __restrict__ part_ml, int* __restrict__ arrivals, int Hq, int Hkv, int BS,
                        int bs_shift, float scale, int window, int split_len_arg, int n_splits,
-                       int group_pad_log2, FusedQkv fz, int out_tiled) {
+                       int group_pad_log2, FusedQkv fz, int out_tiled, float softcap) {
     static_assert(!FUSED || (RT == 1 && QK_K32), "the fused form: one row tile, head sizes in steps of 32");
     // One piece of LDS: the waves' V tiles while the keys are walked; afterwards, with key
     // splits, what the four waves of the workgroup have gathered, to be combined.
@@ -605,6 +617,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
     }
 
     const float c2 = scale * 1.44269504088896340736f;   // scores to base 2
+    const SoftCap capped(scale, softcap);
     const size_t page_stride = (size_t)Hkv * BS * D;
     const bf16* k_base = k_pool + (size_t)kvh * BS * D;
     const bf16* v_base = v_pool + (size_t)kvh * BS * D;
@@ -700,6 +713,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 sv[r] = s[r];
+                if (capped.a != 0.f) sv[r] = capped(sv[r]);
                 if constexpr (MASKED) {
                     const int key = key0 + 4 * kb + r;
                     bool seen = key <= row_pos[rt] && key < hi && key >= lo_seen;
@@ -989,7 +1003,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
                                         const int* positions, const int* row_blocks, int n_row_blocks,
                                         void* out, float* part_o, float* part_ml, int* arrivals, int N,
                                         int Hq, int Hkv, int BS, float scale, int window, int split_len,
-                                        int n_splits, int row_tiles, int group_pad_log2, int out_tiled,
+                                        int n_splits, int row_tiles, int group_pad_log2, int out_tiled, float softcap,
                                         hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
     if (out_tiled && (out_tiled < 0 || N > out_tiled || out_tiled > 64 || (Hq * D) % 32)) return (int)hipErrorInvalidValue;
@@ -1001,7 +1015,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     const int G = Hq / Hkv;
     if ((1 << group_pad_log2) < (G < 16 ? G : 16) || group_pad_log2 > 4) return (int)hipErrorInvalidValue;
     if (n_splits > 256) return (int)hipErrorInvalidValue;
-    if (!(scale > 0.f)) return (int)hipErrorInvalidValue;        // the maximum is taken of the raw scores
+    if (!(scale > 0.f) || softcap < 0.f) return (int)hipErrorInvalidValue;   // the maximum is taken of the raw scores
     const long tasks = (long)n_row_blocks * Hkv * ((G + 15) / 16);
     if (tasks > 0x7fffffffL) return (int)hipErrorInvalidValue;
     const FusedQkv fz{};
@@ -1011,7 +1025,7 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
         for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
 #define SOC_MFMA_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, row_blocks, n_row_blocks, (bf16*)out, part_o, part_ml, arrivals, Hq, Hkv, BS, bs_shift, \
-        scale, window, split_len, n_splits, group_pad_log2, fz, out_tiled
+        scale, window, split_len, n_splits, group_pad_log2, fz, out_tiled, softcap
     // Row tiles beyond what the registers hold at this head size are refused: two up to head
     // size 128, four up to 64.
     const bool tp = bs_shift >= 4;
@@ -1080,7 +1094,7 @@ SOC_EXPORT int soc_paged_attention_decode_fused(const void* qkv, int row_heads, 
             for (bs_shift = 0; (1 << bs_shift) < BS; ++bs_shift) {}
 #define SOC_FUSED_ARGS (const bf16*)nullptr, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, (const int*)nullptr, N, (bf16*)out, part_o, part_ml, arrivals, Hq, Hkv, BS, bs_shift, \
-        scale, window, split_len, n_splits, group_pad_log2, fz, out_tiled
+        scale, window, split_len, n_splits, group_pad_log2, fz, out_tiled, 0.f
         if (bs_shift >= 4)
             hipLaunchKernelGGL((paged_attn_mfma_kernel<1, true, true>), grid, dim3(256), 0, stream, SOC_FUSED_ARGS);
         else
@@ -1145,7 +1159,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                           bf16* __restrict__ out, int Hq, int Hkv, int BS, int bs_shift, float scale,
                           int window, int group_pad_log2, int keep_first, int sink, const float* __restrict__ sinks,
                           const bf16* __restrict__ mean_k, const bf16* __restrict__ mean_v,
-                          const int* __restrict__ mean_table, int mean_table_width, int pool) {
+                          const int* __restrict__ mean_table, int mean_table_width, int pool, float softcap) {
     static_assert(D <= 128, "one key pair per thread");
     static_assert(KS == 1 || (KS == 2 && M32), "key halves come with the 32-row products");
     constexpr int PF_TILE_ELEMS = PF_K_ELEMS + PF_V_ELEMS;          // one K tile and one V^T tile
@@ -1202,6 +1216,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
     const int wave_hi_pos = min(khi, wave_lo_pos + tokens_per_wave) - 1;
     const bool wave_has_rows = wtok0 < ntok;
     const float c2 = scale * 1.44269504088896340736f;               // to base 2
+    const SoftCap capped(scale, softcap);
     const int means_lo = pool > 0 ? blocks_before(wave_lo_pos) : 0; // entries that all / any of the wave's rows see
     const int means_hi = pool > 0 ? blocks_before(wave_hi_pos) : 0;
 
@@ -1364,6 +1379,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 t[r] = r < 4 ? s0[r & 3] : s1[r & 3];
+                if (capped.a != 0.f) t[r] = capped(t[r]);
                 if constexpr (MASKED) {
                     const int key = key0 + 8 * kb + r;
                     bool seen = key <= row_pos[rt];
@@ -1431,6 +1447,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
         float mx = -INFINITY;                               // of the raw scores: the scale is positive
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
+            if (capped.a != 0.f) sc[i] = capped(sc[i]);
             if constexpr (MASKED) {
                 const int key = key0 + 16 * (i / 8) + 8 * g32 + i % 8;
                 bool seen = key <= row_pos32;
@@ -1637,8 +1654,9 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
                                            void* out, int N, int Hq, int Hkv, int BS, float scale,
                                            int window, int row_tiles, int group_pad_log2, int keep_first, int sink,
                                            const float* sinks, const void* mean_k, const void* mean_v, const int* mean_table,
-                                           int mean_table_width, int pool, hipStream_t stream) {
+                                           int mean_table_width, int pool, float softcap, hipStream_t stream) {
     if (N <= 0 || n_row_blocks <= 0) return 0;
+    if (softcap < 0.f) return (int)hipErrorInvalidValue;
     if (Hkv < 1 || Hq % Hkv || BS < 1 || keep_first < 0) return (int)hipErrorInvalidValue;
     if (row_tiles == 64 && (keep_first > 0 && window > 0)) return (int)hipErrorInvalidValue;   // no kept keys with key halves
     if (sink < 0 || sink > 2 || (sink == 2 && !sinks)) return (int)hipErrorInvalidValue;
@@ -1656,7 +1674,7 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
     if constexpr (D <= 128) {
 #define SOC_PF_ARGS (const bf16*)q, (const bf16*)k_pool, (const bf16*)v_pool, block_table, table_width, \
         token_rows, positions, row_blocks, (bf16*)out, Hq, Hkv, BS, bs_shift, scale, window, group_pad_log2, \
-        keep_first, sink, sinks, (const bf16*)mean_k, (const bf16*)mean_v, mean_table, mean_table_width, pool
+        keep_first, sink, sinks, (const bf16*)mean_k, (const bf16*)mean_v, mean_table, mean_table_width, pool, softcap
         const bool pair = bs_shift >= 1;
 #define SOC_PF_LAUNCH(RT_, M32_, KS_)                                                                            \
     do {                                                                                                    \

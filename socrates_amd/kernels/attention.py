@@ -166,7 +166,7 @@ class Attention:
             return split_len, n_splits
         return plan_key_splits(n_blocks, n_kv_heads, group, max_keys, self.split_target_waves, self.split_min_keys)
 
-    def _wave_attention(self, lib, q, slot, ctx, out, scale, w, rt, gpl, which):
+    def _wave_attention(self, lib, q, slot, ctx, out, scale, w, rt, gpl, which, softcap=0.0):
         """The per-wave MFMA kernel with key splits and merge, for all sequences of the step
         or for its short ones (``which``), on the current stream."""
         N, Hq, D = q.shape
@@ -192,7 +192,7 @@ class Attention:
             c_int(slot.block_table.shape[1]), _ptr(ctx.token_rows), _ptr(ctx.positions), _ptr(blocks),
             c_int(n_blocks), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(self._split_count), c_int(N),
             c_int(Hq), c_int(Hkv), c_int(slot.block_size), c_float(scale), c_int(w), c_int(split_len), c_int(n_splits),
-            c_int(rt), c_int(gpl), c_int(0), self._stream()), "paged_attention (mfma)")
+            c_int(rt), c_int(gpl), c_int(0), c_float(softcap), self._stream()), "paged_attention (mfma)")
 
     def rope_table(self, inv_freq, first_pos, n_pos, out=None):
         """Cosines and sines of positions first_pos .. first_pos + n_pos - 1 with the rotation
@@ -280,7 +280,8 @@ class Attention:
         cache slot, whose pages of means hold one mean key and value per block of ``slot.pool`` positions: a token sees
         the blocks that end before its window begins, in the same softmax). Such a layer,
         and one whose scale is not positive, goes to the kernel that computes scores on the
-        vector units, in either dtype; the MFMA kernels take plain scores only."""
+        vector units, in either dtype; the MFMA kernels take plain scores, a soft cap, and (the kernel for prompt
+        portions) kept first keys, pooled blocks and sinks."""
         N, Hq, D = q.shape
         self._want(q, "q", self.dtype)
         Hkv = slot.k.shape[1]
@@ -317,14 +318,15 @@ class Attention:
                 self._check_slot(means, Hkv, D)
                 if means.block_size != slot.block_size:
                     raise KernelError("attention: the pages of means hold as many entries as the tokens' pages")
-        plain = softcap == 0.0 and sinks is None and slopes is None and scale > 0 and keep_first == 0 and not pool
+        # (a soft cap alone is a term of all kernels on the matrix cores: such a layer goes where a plain one goes)
+        plain = sinks is None and slopes is None and scale > 0 and keep_first == 0 and not pool
         # The kernel that shares K and V tiles among four waves also takes kept first keys, the means of pooled
         # blocks, and one more weight in a row's sum (of score 0: ``sinks`` all zero, which ``terms["zero_sink"]`` says
         # without a look at the device; or of the head's own score); the per-wave kernel with key splits does not,
         # so a step with a long portion sends all its rows to the former (behind a window no row walks far), and
         # steps of short portions and decoded tokens go to the vector-unit kernel.
         zero_sink = bool(terms and terms.get("zero_sink")) and sinks is not None
-        windowed = (softcap == 0.0 and slopes is None and scale > 0
+        windowed = (slopes is None and scale > 0
                     and (keep_first > 0 or sinks is not None or pool > 0))
         if self.dtype == torch.bfloat16 and self.attention_mfma and (plain or windowed):
             gpl = max(0, (min(G, 16) - 1).bit_length())
@@ -387,17 +389,18 @@ class Attention:
                     c_float(scale), c_int(w), c_int(rt), c_int(gpl), c_int(keep_first),
                     c_int(0 if sinks is None else (1 if zero_sink else 2)), _ptr(sinks),
                     _ptr(means.k if pool else None), _ptr(means.v if pool else None), _ptr(means.block_table if pool else None),
-                    c_int(means.block_table.shape[1] if pool else 0), c_int(pool), self._stream()), "paged_attention (prefill)")
+                    c_int(means.block_table.shape[1] if pool else 0), c_int(pool), c_float(softcap), self._stream()),
+                    "paged_attention (prefill)")
                 if mixed:
                     # after the long ones, on the same stream: side by side on a second stream
                     # was measured and is slower (35.4 ms against 32.3 ms per mixed step at 8B sizes)
-                    self._wave_attention(lib, q, slot, ctx, out, scale, w, 1, gpl, "short")
+                    self._wave_attention(lib, q, slot, ctx, out, scale, w, 1, gpl, "short", softcap)
                 return out
             if not windowed:
                 rt = self.attention_row_tiles or 1
                 rt = min(rt, 4 if D <= 64 else (2 if D <= 128 else 1))      # what the kernel is built with
                 self.last_attention_kernel = ("wave", rt)
-                self._wave_attention(lib, q, slot, ctx, out, scale, w, rt, gpl, None)
+                self._wave_attention(lib, q, slot, ctx, out, scale, w, rt, gpl, None, softcap)
                 return out
         self.last_attention_kernel = ("tokens", 0)
         max_keys = ctx.max_ctx_len if not w else min(w + keep_first, ctx.max_ctx_len)

@@ -142,6 +142,51 @@ def test_prepare_kernel_with_a_norm_behind_the_rotation(kernel_sets, dtype, norm
     assert float(outs[0][1][0].float().abs().max()) == 7.0                  # the null page is nobody's
 
 
+@pytest.mark.parametrize("P,G", [(64, 2), (128, 4), (48, 1), (32, 8)])
+@pytest.mark.parametrize("row_tiles", [None, 1, 2, 32, 64])
+@pytest.mark.parametrize("window,keep", [(None, 0), (90, 5)])
+def test_a_soft_cap_in_the_attention_kernels_on_the_matrix_cores(kernel_sets, P, G, row_tiles, window, keep):
+    """bfloat16 scores under a soft cap that bites (scores of several times the cap's size): long portions through every
+    form of the kernel that shares its key tiles among four waves (one from position 0, one behind 300 cached tokens,
+    also behind a window with kept first keys), single tokens behind long contexts through the per-wave kernel with
+    its key splits, against the stand-in."""
+    from socrates_amd.cache.manager import PagedSlot
+    ops, dt = kernel_sets["bfloat16"], torch.bfloat16
+    if row_tiles in (32, 64) and P % 32:
+        pytest.skip("32-row products take head sizes in steps of 32")
+    if row_tiles == 64 and keep:
+        pytest.skip("no kept keys with the keys in two halves")
+    ref = TorchKernels(dt, DEV)
+    g = torch.Generator(device="cpu").manual_seed(P + G)
+    Hkv, bs, pages = 2, 16, 48
+    Hq = Hkv * G
+    table = torch.arange(1, 1 + 5 * pages, dtype=torch.int32, device=DEV).view(5, pages)
+    table = torch.cat([table, torch.zeros(1, pages, dtype=torch.int32, device=DEV)]).contiguous()
+    slot = PagedSlot((torch.randn(1 + 5 * pages, Hkv, bs, P, generator=g) * 0.8).to(dt).to(DEV),
+                     torch.randn(1 + 5 * pages, Hkv, bs, P, generator=g).to(dt).to(DEV), table, bs, window)
+    terms = {"softcap": 3.0}
+    if keep:
+        terms["keep_first"] = keep
+    for lengths, rows, starts in (([700, 1, 230, 1, 17], [0, 1, 2, 3, 4], [0, 59, 300, 5, 140]),
+                                  ([1, 1, 1, 1], [0, 1, 2, 4], [699, 0, 530, 17])):
+        ctx = _ctx(lengths, rows, starts, DEV)
+        q = torch.randn(ctx.n_tokens, Hq, P, generator=g).to(dt).to(DEV)
+        want = ref.paged_attention(q, slot, ctx, 1.0, window, terms=terms)
+        uncapped = ref.paged_attention(q, slot, ctx, 1.0, window, terms={k: v for k, v in terms.items() if k != "softcap"} or None)
+        assert float((want.float() - uncapped.float()).abs().max()) > 0.2          # the cap matters here
+        ops.attention_row_tiles = row_tiles if max(lengths) > 1 else None
+        try:
+            got = ops.paged_attention(q, slot, ctx, 1.0, window, terms=terms)
+            kernel = ops.last_attention_kernel
+        finally:
+            ops.attention_row_tiles = None
+        if max(lengths) > 1 and row_tiles:
+            assert kernel == ("workgroup", row_tiles)
+        elif not keep:
+            assert kernel[0] == "wave"
+        _close(got, want, "bfloat16", f"soft cap, window {window}, {keep} kept, row tiles {row_tiles} ({kernel})")
+
+
 @pytest.mark.parametrize("E,top,count,keep,group_top", [(12, 3, 4, 2, 2), (8, 8, 8, 8, 2), (6, 1, 1, 1, 2), (9, 2, 3, 1, 3), (200, 6, 20, 7, 2),
                                                         (256, 8, 1, 1, 1), (10, 4, 5, 3, 1)])
 def test_choice_of_experts_kernel(kernel_sets, E, top, count, keep, group_top):
