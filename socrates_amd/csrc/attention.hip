@@ -710,10 +710,13 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 s = qk_mfma(k_ok ? kf.v[kk] : make_uint4(0u, 0u, 0u, 0u), qf[rt][kk], s);
             float sv[4];
             float mx = -INFINITY;                           // of the raw scores: the scale is positive
+            if (capped.a != 0.f) {                          // (one branch on a scalar for the tile's scores, not a select each)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) s[r] = capped(s[r]);
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 sv[r] = s[r];
-                if (capped.a != 0.f) sv[r] = capped(sv[r]);
                 if constexpr (MASKED) {
                     const int key = key0 + 4 * kb + r;
                     bool seen = key <= row_pos[rt] && key < hi && key >= lo_seen;
@@ -1376,10 +1379,13 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             }
             float t[8];
             float mx = -INFINITY;                           // of the raw scores: the scale is positive
+            if (capped.a != 0.f) {                          // (one branch on a scalar for the tile's scores, not a select each)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) { s0[r] = capped(s0[r]); s1[r] = capped(s1[r]); }
+            }
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
                 t[r] = r < 4 ? s0[r & 3] : s1[r & 3];
-                if (capped.a != 0.f) t[r] = capped(t[r]);
                 if constexpr (MASKED) {
                     const int key = key0 + 8 * kb + r;
                     bool seen = key <= row_pos[rt];
@@ -1445,9 +1451,12 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                                                          *reinterpret_cast<const bf16x8_t*>(&qf32[t]), sc, 0, 0, 0);
         }
         float mx = -INFINITY;                               // of the raw scores: the scale is positive
+        if (capped.a != 0.f) {                              // (one branch on a scalar for the tile's scores, not a select each)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sc[i] = capped(sc[i]);
+        }
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            if (capped.a != 0.f) sc[i] = capped(sc[i]);
             if constexpr (MASKED) {
                 const int key = key0 + 16 * (i / 8) + 8 * g32 + i % 8;
                 bool seen = key <= row_pos32;

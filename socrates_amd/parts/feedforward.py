@@ -37,6 +37,10 @@ class SwiGLU:
     takes_projection = True     # the block may supply the last product
     takes_norm_owed = True      # x goes to one product only
 
+    def rows_as_they_are(self):
+        """The activation goes to a product that reads plain rows (a caller's own ``project``): keep the rows' layout."""
+        self._free_layout = {}
+
     def forward(self, x, ctx=None, project=None):
         act = self.ops.linear_swiglu(x, self.w_gate_up, self.interleave, **self._free_layout)
         if project is not None:

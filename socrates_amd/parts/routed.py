@@ -57,6 +57,8 @@ class RoutedExperts:
         if spec.shared is not None:
             own = {k[len("shared."):]: v for k, v in tensors.items() if k.startswith("shared.") and k != "shared.sg"}
             self.shared = build_part(spec.shared, own, ops)
+            if hasattr(self.shared, "rows_as_they_are"):
+                self.shared.rows_as_they_are()
 
     def forward(self, x, ctx=None):
         s, ops = self.spec, self.ops
@@ -66,7 +68,12 @@ class RoutedExperts:
         how = {} if plain else dict(scoring=s.scoring, group_top=s.group_top, scale=s.scale)
         experts, weights = ops.moe_route(logits[:, :E] if s.shared_gate else logits, self.correction, s.top, s.n_groups,
                                          s.keep_groups, s.renorm_eps, **how)
-        extra = self.shared.forward(x) if self.shared is not None else None
+        extra = None
+        if self.shared is not None and getattr(self.shared, "takes_projection", False):
+            # (a feed-forward that would hand partial sums to a norm: here its last product is whole)
+            extra = self.shared.forward(x, project=lambda act, w: ops.linear(act, w))
+        elif self.shared is not None:
+            extra = self.shared.forward(x)
         limit, slope, shift = self.form
         more = {}
         if shift != 1.0:
