@@ -414,7 +414,7 @@ struct FusedQkv {
     bf16* v_pool_w;
 };
 
-// A soft cap on the scores inside the kernels on the matrix cores: the raw score t becomes (cap / scale) tanh(t scale /
+// A soft cap on the scores inside the kernels on the matrix cores (their CAP forms): the raw score t becomes (cap / scale) tanh(t scale /
 // cap), so that what follows (the maximum, times scale log2 e) works on it as on a raw score. tanh(x) =
 // 1 - 2 / (exp2(2 x log2 e) + 1). ``a`` = cap / scale (0: no cap), ``b`` = 2 log2 e scale / cap.
 struct SoftCap {
@@ -426,7 +426,7 @@ struct SoftCap {
     }
 };
 
-template <int RT, bool TP, bool FUSED = false>
+template <int RT, bool TP, bool FUSED = false, bool CAP = false>
 __global__ void __launch_bounds__(256)
 paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
                        const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
@@ -710,7 +710,7 @@ paged_attn_mfma_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_po
                 s = qk_mfma(k_ok ? kf.v[kk] : make_uint4(0u, 0u, 0u, 0u), qf[rt][kk], s);
             float sv[4];
             float mx = -INFINITY;                           // of the raw scores: the scale is positive
-            if (capped.a != 0.f) {                          // (one branch on a scalar for the tile's scores, not a select each)
+            if constexpr (CAP) {                            // (a form of its own: a layer without a cap pays nothing)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) s[r] = capped(s[r]);
             }
@@ -1034,7 +1034,10 @@ SOC_EXPORT int soc_paged_attention_mfma(const void* q, const void* k_pool, const
     const bool tp = bs_shift >= 4;
 #define SOC_MFMA_LAUNCH(RT_)                                                                          \
     do {                                                                                              \
-        if (tp) hipLaunchKernelGGL((paged_attn_mfma_kernel<RT_, true>), grid, dim3(256), 0, stream, SOC_MFMA_ARGS); \
+        if (softcap > 0.f) {                                                                          \
+            if (tp) hipLaunchKernelGGL((paged_attn_mfma_kernel<RT_, true, false, true>), grid, dim3(256), 0, stream, SOC_MFMA_ARGS); \
+            else hipLaunchKernelGGL((paged_attn_mfma_kernel<RT_, false, false, true>), grid, dim3(256), 0, stream, SOC_MFMA_ARGS);   \
+        } else if (tp) hipLaunchKernelGGL((paged_attn_mfma_kernel<RT_, true>), grid, dim3(256), 0, stream, SOC_MFMA_ARGS); \
         else hipLaunchKernelGGL((paged_attn_mfma_kernel<RT_, false>), grid, dim3(256), 0, stream, SOC_MFMA_ARGS);   \
     } while (0)
     if (row_tiles == 1) {
@@ -1153,7 +1156,7 @@ constexpr int PF_MEAN = -(1 << 30);
 // at the end the two partial results are combined through LDS. Twice the waves for the same
 // number of workgroups: for launches whose workgroups are too few, or too uneven (a prompt
 // from its start: the last block sees all keys, the first none), to fill the GPU otherwise.
-template <int RT, bool PAIR, bool M32, int KS>
+template <int RT, bool PAIR, bool M32, int KS, bool CAP = false>
 __global__ void __launch_bounds__(256 * KS)
 paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_pool,
                           const bf16* __restrict__ v_pool, const int* __restrict__ block_table,
@@ -1379,7 +1382,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
             }
             float t[8];
             float mx = -INFINITY;                           // of the raw scores: the scale is positive
-            if (capped.a != 0.f) {                          // (one branch on a scalar for the tile's scores, not a select each)
+            if constexpr (CAP) {                            // (a form of its own: a layer without a cap pays nothing)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) { s0[r] = capped(s0[r]); s1[r] = capped(s1[r]); }
             }
@@ -1451,7 +1454,7 @@ paged_attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k
                                                          *reinterpret_cast<const bf16x8_t*>(&qf32[t]), sc, 0, 0, 0);
         }
         float mx = -INFINITY;                               // of the raw scores: the scale is positive
-        if (capped.a != 0.f) {                              // (one branch on a scalar for the tile's scores, not a select each)
+        if constexpr (CAP) {                                // (a form of its own: a layer without a cap pays nothing)
 #pragma unroll
             for (int i = 0; i < 16; ++i) sc[i] = capped(sc[i]);
         }
@@ -1687,7 +1690,10 @@ SOC_EXPORT int soc_paged_attention_prefill(const void* q, const void* k_pool, co
         const bool pair = bs_shift >= 1;
 #define SOC_PF_LAUNCH(RT_, M32_, KS_)                                                                            \
     do {                                                                                                    \
-        if (pair) hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, true, M32_, KS_>), dim3((unsigned)groups), dim3(256 * KS_), 0, stream, SOC_PF_ARGS); \
+        if (softcap > 0.f) {                                                                                \
+            if (pair) hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, true, M32_, KS_, true>), dim3((unsigned)groups), dim3(256 * KS_), 0, stream, SOC_PF_ARGS); \
+            else hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, false, M32_, KS_, true>), dim3((unsigned)groups), dim3(256 * KS_), 0, stream, SOC_PF_ARGS);     \
+        } else if (pair) hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, true, M32_, KS_>), dim3((unsigned)groups), dim3(256 * KS_), 0, stream, SOC_PF_ARGS); \
         else hipLaunchKernelGGL((paged_attn_prefill_kernel<RT_, false, M32_, KS_>), dim3((unsigned)groups), dim3(256 * KS_), 0, stream, SOC_PF_ARGS);     \
     } while (0)
         if (row_tiles == 1) SOC_PF_LAUNCH(1, false, 1);
