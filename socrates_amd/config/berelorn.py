@@ -223,9 +223,11 @@ class BerelornConfig:
         d, eps = self.width, self.norm_eps
         layers = [_thaw(x) for x in self.layers]
         norm = RMSNormSpec(d, eps, tensor="")
-        blocks, order = [], []
+        blocks, order, ignorable = [], [], []
         for i, layer in enumerate(layers):
             ffn = self._ffn(layer.get("mlp"))
+            if ffn is None:                 # (a file may hold the norms of a feed-forward that the layer lacks)
+                ignorable += [f"l{i}.norm2", f"l{i}.norm2b"]
             blocks.append(BlockSpec(mixer=self._mixer(i, layers), ffn=ffn, norm1=norm, post_norm1=norm,
                                     norm2=None if ffn is None else norm, post_norm2=None if ffn is None else norm,
                                     prefix=f"l{i}.", names=_NAMES, arrangement="sandwich"))
@@ -234,7 +236,7 @@ class BerelornConfig:
         return ModelPlan(
             architecture=self.architecture, vocab_size=self.vocab, hidden=d, layers=tuple(blocks), order=tuple(order),
             final_norm=norm, embedding_name="embed", final_norm_prefix="final.norm", head_name=None,
-            eos_token_ids=self.eos_token_ids, embedding_scale=self.embedding_scale)
+            eos_token_ids=self.eos_token_ids, ignorable=tuple(ignorable), embedding_scale=self.embedding_scale)
 
     # ---- byte and flop counts ---------------------------------------------------------
     def _shares(self, plan, of):

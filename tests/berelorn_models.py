@@ -95,7 +95,7 @@ def drawn_model(seed):
         dims = rng.choice([r for r in (0, 2, 4, 8, 12, 16, 24, 40, 64) if r <= dim])
         if not dims:
             return None
-        scaling = None if rng.random() < 0.3 else (rng.choice([2.0, 4.0, 8.0]), rng.choice([16, 64, 2048]), rng.choice([4.0, 32.0]),
+        scaling = None if rng.random() < 0.3 else (rng.choice([3.0, 4.0, 8.0]), rng.choice([16, 64, 4096]), rng.choice([4.0, 16.0]),
                                                    rng.choice([0.5, 1.0, 2.0]))
         return rot(dims, rng.choice([100.0, 10000.0, 1e6]), scaling)
 

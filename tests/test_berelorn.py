@@ -54,6 +54,7 @@ def test_plan_follows_the_configuration(folders):
     assert needs[2] == PagedKV(4, 16, None, 0) and needs[3] is None
     assert [(s.layer, s.cache, s.write) for s in plan.order] == [(0, 0, True), (1, 1, True), (2, 2, True), (3, 1, False), (4, 4, True)]
     assert plan.head_name is None and plan.embedding_scale == 6.0
+    assert set(plan.ignorable) == {"l1.norm2", "l1.norm2b", "l4.norm2", "l4.norm2b"}
     names = expected_tensors(plan)
     want = tensor_shapes(MODELS["A"])
     assert set(names) == set(want)

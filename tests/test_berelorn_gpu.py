@@ -336,6 +336,34 @@ def test_a_wider_model_with_long_prompts(tmp_path, kernel_sets, dtype):
 
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
+def test_a_model_of_a_thousand_columns(tmp_path, kernel_sets, dtype):
+    """Width 1,024 and heads of 128: matrices large enough for the products' other forms (weights read by tile, the
+    sweeps, the library beyond 16 rows, the experts' large tiles), a state of 128 x 128, two maps of 128 over values of
+    64, prompts of up to 300 tokens decoded at the end and mixed, through captured decode steps."""
+    position = rot(64, 500000.0, (8.0, 4096, 16.0, 2.0))
+    cfg = model(1024, 2000, [memory(4, 128, 128, 18.0),
+                             differential(4, 2, 128, 64, size=64, keep=6, rotation=position, diff=0.35, scale=0.09),
+                             keyed(8, 4, 128, rot(128, 1e6, (4.0, 1024, 16.0, 1.0)), scale=6.0, softcap=20.0),
+                             differential(4, 2, 128, 64, size=150, keep=2, rotation=position, diff=0.6, scale=0.09, kv_from=1)],
+                [moe(8, 2, 512, count=4, keep=2, scale=1.8, shared=768), moe(4, 1, 1024), None, moe(8, 3, 256, count=2, keep=2, shared=256)],
+                embedding=10.0)
+    folder = write_model(tmp_path / "m", cfg, seed=9)
+    prompts = random_prompts([300, 120, 33], cfg["vocab"], seed=10)
+    want = oracle(folder, prompts)
+    for name, steps in (("tail", trace_tail_decode(prompts, 24)), ("mixed", trace_mixed(prompts, seed=11))):
+        runner = make_runner(folder, kernel_sets[dtype], max_rows=4, max_len=320, block_size=16)
+        runner.enable_graphs(4)
+        got = replay(runner, steps)
+        if dtype == "float32":
+            for i in range(len(prompts)):
+                compare(got[f"r{i}"], want[i], TOL[dtype], f"{name} {dtype} request {i}")
+        else:
+            rounded = replay(make_runner(folder, TorchKernels(torch.bfloat16, "cpu"), max_rows=4, max_len=320, block_size=16), steps)
+            for i in range(len(prompts)):
+                judged_in_bfloat16(got[f"r{i}"], want[i], rounded[f"r{i}"], f"{name} request {i}")
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
 def test_edges_and_long_decoding(tmp_path, kernel_sets, dtype):
     """A window of 6 with 3 kept tokens, read again by a layer behind a window of 4 with 5 kept (in float32 under a
     sharp softmax, so the key at an edge often carries the weight; in bfloat16 a flatter one, where rounding moves
