@@ -14,45 +14,62 @@ __device__ __forceinline__ float mem_logsigmoid(float u) { return fminf(u, 0.f) 
 // gates: float32 [N, 2 H], the logits of the input gates (columns 0 .. H - 1) and of the forget gates (H .. 2 H - 1);
 // bias float32 [2 H]. i = cap tanh((z_i + b_i) / cap), f = logsigmoid(cap tanh((z_f + b_f) / cap)). Per sequence and
 // head, from the maximum m that the row's state holds (at offset + head): m' = max(f + m, i), keep = exp(f + m - m'),
-// take = exp(i - m'); maxima, keep and take are float32 [N, H]; the row's maximum is left for the next step. One wave
-// per (sequence, head) walks 64 tokens at a time: a token is the map m -> max(F + m, I) with (F, I) = (f, i), maps
-// compose as (F1, I1) then (F2, I2) = (F1 + F2, max(I1 + F2, I2)), and a scan over the lanes composes them in order.
-__global__ void __launch_bounds__(64)
+// take = exp(i - m'); maxima, keep and take are float32 [N, H]; the row's maximum is left for the next step. A token is
+// the map m -> max(F + m, I) with (F, I) = (f, i), and maps compose as (F1, I1) then (F2, I2) = (F1 + F2, max(I1 + F2,
+// I2)). One workgroup per (sequence, head), of 1 to 16 waves (more for long portions), walks blockDim.x tokens per
+// round: every wave composes its 64 tokens' maps in order by a scan over its lanes, the waves' totals meet in LDS,
+// and a token's maximum is the map of all tokens of the round before it applied to what the rounds before left.
+struct GateMap { float F, I; };
+__device__ __forceinline__ GateMap then(GateMap a, GateMap b) { return GateMap{a.F + b.F, fmaxf(a.I + b.F, b.I)}; }
+
+__global__ void __launch_bounds__(1024)
 memory_scan_kernel(const float* __restrict__ gates, const float* __restrict__ bias, float cap, int H,
                    float* __restrict__ state, size_t stride, int offset, const int* __restrict__ seq_qstart,
                    const int* __restrict__ seq_rows, float* __restrict__ maxima, float* __restrict__ keep,
                    float* __restrict__ take) {
-    const int seq = blockIdx.y, head = blockIdx.x, lane = threadIdx.x;
+    __shared__ float totals[2][16][2];
+    const int seq = blockIdx.y, head = blockIdx.x;
+    const int wave = threadIdx.x / SOC_WAVE, lane = threadIdx.x % SOC_WAVE, n_waves = blockDim.x / SOC_WAVE;
     const int lo = seq_qstart[seq], hi = seq_qstart[seq + 1];
-    if (lo >= hi) return;
+    if (lo >= hi) return;                                   // (the whole workgroup: no barrier is left waiting)
     float* held = state + (size_t)seq_rows[seq] * stride + offset + head;
     float carry = *held;
     const float bi = bias[head], bf = bias[H + head], inv_cap = 1.f / cap;
-    for (int n0 = lo; n0 < hi; n0 += SOC_WAVE) {
-        const int n = n0 + lane;
+    int buf = 0;
+    for (int n0 = lo; n0 < hi; n0 += blockDim.x, buf ^= 1) {
+        const int n = n0 + threadIdx.x;
         const bool in = n < hi;
         float gi = -INFINITY, gf = 0.f;                    // (behind the end: the map that changes nothing)
         if (in) {
             gi = cap * tanhf((gates[(size_t)n * 2 * H + head] + bi) * inv_cap);
             gf = mem_logsigmoid(cap * tanhf((gates[(size_t)n * 2 * H + H + head] + bf) * inv_cap));
         }
-        float F = gf, I = gi;
+        GateMap mine{gf, gi};                               // becomes the map of the wave's tokens up to this one
 #pragma unroll
         for (int d = 1; d < SOC_WAVE; d <<= 1) {
-            const float Fp = __shfl_up(F, d, SOC_WAVE), Ip = __shfl_up(I, d, SOC_WAVE);
-            if (lane >= d) { I = fmaxf(Ip + F, I); F = Fp + F; }
+            const GateMap before{__shfl_up(mine.F, d, SOC_WAVE), __shfl_up(mine.I, d, SOC_WAVE)};
+            if (lane >= d) mine = then(before, mine);
         }
-        const float m = fmaxf(F + carry, I);
+        if (lane == SOC_WAVE - 1) { totals[buf][wave][0] = mine.F; totals[buf][wave][1] = mine.I; }
+        __syncthreads();
+        GateMap ahead{0.f, -INFINITY}, whole{0.f, -INFINITY};     // the waves before this one; all waves of the round
+        for (int w = 0; w < n_waves; ++w) {
+            const GateMap t{totals[buf][w][0], totals[buf][w][1]};
+            if (w < wave) ahead = then(ahead, t);
+            whole = then(whole, t);
+        }
+        const float start = fmaxf(ahead.F + carry, ahead.I);      // the maximum in front of this wave's first token
+        const float m = fmaxf(mine.F + start, mine.I);
         float before = __shfl_up(m, 1, SOC_WAVE);
-        if (lane == 0) before = carry;
+        if (lane == 0) before = start;
         if (in) {
             maxima[(size_t)n * H + head] = m;
             keep[(size_t)n * H + head] = expf(gf + before - m);
             take[(size_t)n * H + head] = expf(gi - m);
         }
-        carry = __shfl(m, SOC_WAVE - 1, SOC_WAVE);
+        carry = fmaxf(whole.F + carry, whole.I);
     }
-    if (lane == 0) *held = carry;
+    if (threadIdx.x == 0) *held = carry;
 }
 
 // prep [N, 3, H D] float32: q scaled, k times the token's take, and the token's keep for every key channel.
@@ -74,11 +91,13 @@ __global__ void memory_prepare_kernel(const T* __restrict__ x, int ld, int col_q
 
 SOC_EXPORT int soc_memory_gates(const float* gates, const float* bias, float cap, const void* x, int ld, int col_q, int col_k,
                                 float q_scale, int H, int D, float* state, long long stride, int offset,
-                                const int* seq_qstart, const int* seq_rows, int n_seqs, int N, float* maxima, float* keep,
-                                float* take, float* prep, int dtype, hipStream_t stream) {
+                                const int* seq_qstart, const int* seq_rows, int n_seqs, int max_q_len, int N, float* maxima,
+                                float* keep, float* take, float* prep, int dtype, hipStream_t stream) {
     if (n_seqs <= 0 || N <= 0 || H <= 0) return 0;
     if (D < 1 || !(cap > 0.f) || n_seqs > 65535 || offset < 0) return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL(memory_scan_kernel, dim3(H, n_seqs), dim3(64), 0, stream, gates, bias, cap, H, state, (size_t)stride,
+    // waves per (sequence, head): one for single tokens and short portions, up to sixteen for long ones
+    const int threads = max_q_len <= 64 ? 64 : max_q_len <= 256 ? 256 : 1024;
+    hipLaunchKernelGGL(memory_scan_kernel, dim3(H, n_seqs), dim3(threads), 0, stream, gates, bias, cap, H, state, (size_t)stride,
                        offset, seq_qstart, seq_rows, maxima, keep, take);
     const size_t total = (size_t)N * H * D;
     const int blocks = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);

@@ -89,7 +89,7 @@ _COMPOSITE_SIGNATURES = {
     "soc_glu_gelu": [P, P, I, I, I, I, P],
 }
 _MEMORY_SIGNATURES = {
-    "soc_memory_gates": [P, P, F, P, I, I, I, F, I, I, P, L, I, P, P, I, I, P, P, P, P, I, P],
+    "soc_memory_gates": [P, P, F, P, I, I, I, F, I, I, P, L, I, P, P, I, I, I, P, P, P, P, I, P],
     "soc_memory_finish": [P, P, P, I, P, I, I, I, F, F, P, I, P],
     "soc_diff_combine": [P, P, I, I, I, I, I, F, F, F, I, P],
 }

@@ -40,7 +40,7 @@ class Memory:
         prep = torch.empty((N, 3, H * D), dtype=torch.float32, device=self.device)
         _check(self._memory().soc_memory_gates(
             _ptr(gates), _ptr(bias), c_float(cap), _ptr(x), c_int(ld), c_int(col_q), c_int(col_k), c_float(q_scale), c_int(H),
-            c_int(D), _ptr(state), stride, c_int(offset), _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), c_int(ctx.n_seqs), c_int(N),
+            c_int(D), _ptr(state), stride, c_int(offset), _ptr(ctx.seq_qstart), _ptr(ctx.seq_rows), c_int(ctx.n_seqs), c_int(max(1, ctx.max_q_len)), c_int(N),
             _ptr(scratch[0]), _ptr(scratch[1]), _ptr(scratch[2]), _ptr(prep), c_int(self.code), self._stream()), "memory_gates")
         return prep, scratch[0]
 

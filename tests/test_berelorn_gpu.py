@@ -59,7 +59,7 @@ def _ctx(lengths, rows, starts, dev):
 # ---- each kernel against its stand-in ----------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("H,D,Dv", [(3, 20, 28), (1, 48, 80), (4, 8, 8), (2, 64, 40), (2, 128, 64), (1, 200, 15), (6, 32, 63)])
-@pytest.mark.parametrize("lengths", [[9, 1, 2, 15], [37, 1, 2, 170]])
+@pytest.mark.parametrize("lengths", [[9, 1, 2, 15], [37, 1, 2, 170], [300, 1, 64, 65], [2300, 17, 1, 1024]])
 def test_matrix_memory_kernels(kernel_sets, dtype, H, D, Dv, lengths):
     """The gates with their running maximum over several sequences of unequal length (more than a wave of tokens among
     them, and single tokens) from maxima that are not zero; the recurrence over prepared q, k and decays with the
@@ -67,6 +67,8 @@ def test_matrix_memory_kernels(kernel_sets, dtype, H, D, Dv, lengths):
     ops, dt = kernel_sets[dtype], DTYPES[dtype]
     ref = TorchKernels(dt, DEV)
     g = torch.Generator(device="cpu").manual_seed(H * D + Dv)
+    if max(lengths) > 1000 and D * Dv > 2000:
+        pytest.skip("the longest portions with the small states only (the stand-in walks token by token)")
     rows, starts = [2, 0, 3, 1], [5, 300, 0, 41]
     ctx = _ctx(lengths, rows, starts, DEV)
     N, ld = ctx.n_tokens, 7 + H * (2 * D + 2 * Dv)
